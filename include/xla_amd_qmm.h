@@ -1,0 +1,183 @@
+/*
+ * xla_amd_qmm.h -- C ABI of libxla_amd_qmm.so: gfx950 (MI355X) kernels for the
+ * quantized-linear operator torch.ops.xla.quantized_matmul and the int8
+ * quantized_matmul_int8 operator of PyTorch/XLA.
+ *
+ * The reference has no native entry point for this path: the operator schema in
+ *   torch_xla/experimental/xla_quantized_matmul.py:7-9
+ *   torch_xla/experimental/custom_kernel.py:1742-1744
+ * is its plugin boundary and the arithmetic is emitted as XLA ops.  Each entry
+ * point below cites the reference statement(s) it replaces.
+ *
+ * Conventions
+ *  - plain pointers and sizes only; every pointer is DEVICE memory unless the
+ *    comment says "host"; all tensors are dense and contiguous (row-major).
+ *  - `stream` is a hipStream_t passed as void* (NULL = default stream).  No
+ *    entry point synchronises the device, allocates or frees device memory, or
+ *    keeps a pointer after it returns.
+ *  - return value: XLA_AMD_QMM_OK or a negative XLA_AMD_QMM_E* code; the text
+ *    of the last error of the calling thread is xla_amd_qmm_last_error().
+ *    No C++ exception crosses this boundary.
+ *  - M = rows of x (tokens), K = in features, N = out features,
+ *    C = block size along K (C == K for per-channel), S = K / C.
+ */
+#ifndef XLA_AMD_QMM_H_
+#define XLA_AMD_QMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XLA_AMD_QMM_ABI_VERSION 1
+
+/* return codes */
+#define XLA_AMD_QMM_OK 0
+#define XLA_AMD_QMM_EINVAL (-1)       /* null pointer, bad size, bad enum */
+#define XLA_AMD_QMM_EUNSUPPORTED (-2) /* shape/dtype the chosen kernel cannot take */
+#define XLA_AMD_QMM_EHIP (-3)         /* HIP launch/runtime error */
+
+/* element types of floating tensors */
+#define XLA_AMD_DT_F32 0
+#define XLA_AMD_DT_BF16 1
+#define XLA_AMD_DT_F16 2
+
+/* float -> int8 conversion of a rounded value outside [-128,127]
+ * (reference: `.to(torch.int8)` with no clamp, xla_quantized_matmul.py:72;
+ * XLA's ConvertElementType saturates, torch's CPU cast wraps modulo 256). */
+#define XLA_AMD_OVERFLOW_SATURATE 0
+#define XLA_AMD_OVERFLOW_WRAP 1
+
+/* memory layout of the int8 weight container handed to the operator */
+#define XLA_AMD_W_NK 0  /* per-channel: [N, K]                 (xla_quantized_matmul.py:88) */
+#define XLA_AMD_W_SCN 1 /* blockwise:   [K/C, C, N]            (xla_quantized_matmul.py:89) */
+
+/* kernels the dispatcher can choose (xla_amd_qmm_dispatch) */
+#define XLA_AMD_KERNEL_GENERIC 0    /* one thread per output, any shape          */
+#define XLA_AMD_KERNEL_SKINNY_MFMA 1 /* weight-streaming GEMV / skinny GEMM       */
+#define XLA_AMD_KERNEL_W8A8_MFMA 2  /* LDS-tiled int8 MFMA GEMM                   */
+#define XLA_AMD_KERNEL_W8A8_GENERIC 3
+
+int xla_amd_qmm_abi_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). Host. */
+const char* xla_amd_qmm_last_error(void);
+
+/*
+ * Bytes of the K-major ("packed") copy of a weight: N*K for bits == 8,
+ * N*K/2 for bits == 4.  Returns 0 for arguments the pack kernel rejects.
+ */
+size_t xla_amd_qmm_packed_bytes(int64_t N, int64_t K, int bits);
+
+/*
+ * One-time re-layout of a weight into the K-major form the streaming kernel
+ * reads.  Replaces the reference's `_xla_cast_int4(w, w.cpu()...tolist())`
+ * (xla_quantized_matmul.py:101-103 -> csrc/ops/cast_int4.cpp:30-39), which
+ * rebuilds the weight as an s4 literal: values are unchanged, only storage.
+ *   src_layout XLA_AMD_W_NK : w is [N, K]       (C ignored, S*C == K)
+ *   src_layout XLA_AMD_W_SCN: w is [S, C, N]
+ *   bits 8: packed[n*K + k] = w(n,k)
+ *   bits 4: values must lie in [-8,7]; packed is [N, K/2] bytes, K % 8 == 0.
+ *           Each aligned group of 8 consecutive k of a row is one 32-bit
+ *           little-endian word; nibble j of the word (bits 4j..4j+3) holds
+ *           (w(n, k0 + P[j]) + 8) with P = {0,2,4,6,1,3,5,7}.
+ */
+int xla_amd_qmm_pack_weight(const int8_t* w, void* packed, int64_t S, int64_t C, int64_t N,
+                            int src_layout, int bits, void* stream);
+
+/*
+ * Weight-only quantized matmul, fast path: streams a K-major weight once and
+ * keeps up to 64 rows of x per pass in MFMA fragments (passes over w repeat
+ * for larger M).  Replaces, with the reference's rounding points,
+ *   per-channel (C == K):  out = F.linear(x, w) * scaler      (:113-114)
+ *   blockwise   (C <  K):  einsum('scn,...sc->...sn'), einsum('sn,...sn->...n') (:122-124)
+ *   zero point:            out -= rowsum/blocksum(x) (x) zp    (:125-133)
+ * x [M,K] (bf16/f16/f32), w_packed from xla_amd_qmm_pack_weight (a per-channel
+ * int8 [N,K] weight already is its own 8-bit packed form), scale [S,N],
+ * zp [S,N] or NULL, out [M,N].
+ * Needs K % 128 == 0 and C % 128 == 0; else XLA_AMD_QMM_EUNSUPPORTED.
+ * out_dt must be the torch promotion of (x_dt, scale_dt).
+ */
+int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packed, const void* scale,
+                                   const void* zp, void* out, int64_t M, int64_t N, int64_t K,
+                                   int64_t C, int bits, int x_dt, int scale_dt, int zp_dt,
+                                   int out_dt, void* stream);
+
+/*
+ * Weight-only quantized matmul for any shape, reading the operator's own
+ * weight layout (one thread per output element; the slow, always-correct path
+ * for shapes the streaming kernel rejects).  Same reference statements and
+ * rounding points as xla_amd_qmm_weight_only_skinny.
+ */
+int xla_amd_qmm_weight_only_generic(const void* x, const int8_t* w, const void* scale,
+                                    const void* zp, void* out, int64_t M, int64_t N, int64_t K,
+                                    int64_t C, int w_layout, int x_dt, int scale_dt, int zp_dt,
+                                    int out_dt, void* stream);
+
+/*
+ * Per-token dynamic activation quantization (`_quantize_tensor`,
+ * xla_quantized_matmul.py:56-73; Pallas `_quantize_array`,
+ * pallas_kernels/quantized_matmul_kernel.py:10-18):
+ *   max = amax(|x|, -1); scale = max / 127; x_q = int8(round_half_even(x / scale))
+ * with every intermediate rounded to x_dt as the reference does op by op.
+ * x [M,K], x_q int8 [M,K], x_scale [M] stored as scale_out_dt (x_dt for the
+ * torch op, f32 for the Pallas variant).  A row of zeros yields x_q = 0,
+ * scale = 0 (the reference leaves this case undefined).
+ * x_sum (nullable) receives sum_k x_q[m,k] as int32 [M]: the factor of the
+ * zero-point term once x has been replaced by its quantized form (:109,:128).
+ */
+int xla_amd_qmm_quantize_per_token(const void* x, int8_t* x_q, void* x_scale, int32_t* x_sum,
+                                   int64_t M, int64_t K, int x_dt, int scale_out_dt,
+                                   int overflow_policy, void* stream);
+
+/*
+ * int8 x int8 -> int32 GEMM with fused scale epilogue.  Replaces
+ *   `_xla_dot_general(x_int, w, (([-1],[-1]),()), preferred_element_type=int32)`
+ *   (xla_quantized_matmul.py:110-111 -> csrc/ops/dot_general.cpp:16-37),
+ *   `out * scaler` (:114), the zero-point term (:125-133), `out * x_scale` (:135)
+ *   and the Pallas matmul_kernel body (pallas_kernels/quantized_matmul_kernel.py:88-124).
+ * x_q int8 [M,K], w int8 [N,K], x_scale [M], w_scale [N]; zp [N] and
+ * x_sum int32 [M] (from xla_amd_qmm_quantize_per_token) both given or both NULL.
+ * Epilogue per element, with round_d = round-to-nearest-even to dtype d:
+ *   v = round_{cvt_dt}(float(acc))
+ *   v = round_{mid_dt}(v * w_scale[n])
+ *   if zp: v = round_{mid_dt}(v - round_{zpo_dt}(round_{zpo_dt}(float(x_sum[m])) * zp[n]))
+ *   v = round_{out_dt}(v * x_scale[m])               -> out[m,n]
+ * (torch converts an integer tensor to the float operand's dtype before it
+ * multiplies, hence cvt_dt and the inner round of x_sum.)
+ * If acc_out != NULL the raw int32 accumulators are also stored to
+ * acc_out [M,N] (parity/debug).  If out == NULL only acc_out is written.
+ * The MFMA kernel needs K % 16 == 0 and 16-byte aligned x_q and w; other
+ * shapes run a one-thread-per-output kernel.
+ * block_m/block_n select the workgroup tile (the role of batch_block_size /
+ * out_block_size, custom_kernel.py:1088-1100): 0,0 = choose by shape;
+ * otherwise one of the pairs xla_amd_qmm_w8a8_tile can return, else
+ * XLA_AMD_QMM_EUNSUPPORTED.
+ */
+int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const void* x_scale,
+                          const void* w_scale, const void* zp, const int32_t* x_sum, void* out,
+                          int32_t* acc_out, int64_t M, int64_t N, int64_t K, int x_scale_dt,
+                          int w_scale_dt, int zp_dt, int cvt_dt, int mid_dt, int zpo_dt,
+                          int out_dt, int block_m, int block_n, void* stream);
+
+/*
+ * Shape-based choice between the kernels (the role of the tuned-table lookup
+ * with fallback in torch_xla/experimental/custom_kernel.py:1088-1106).
+ * Pure host function; returns an XLA_AMD_KERNEL_* id.
+ */
+int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, int bits, int x_dt,
+                         int quantize_activation);
+
+/*
+ * Tile configuration the W8A8 GEMM would use for a shape: fills
+ * tile_mnk[3] = {block_M, block_N, block_K}; the analogue of
+ * get_tuned_block_sizes (pallas_kernels/quantized_matmul_kernel.py:537-555).
+ */
+int xla_amd_qmm_w8a8_tile(int64_t M, int64_t N, int64_t K, int32_t* tile_mnk /* host */);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XLA_AMD_QMM_H_ */

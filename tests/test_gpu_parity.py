@@ -1,0 +1,231 @@
+"""GPU parity: HIP kernels (through the C ABI) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from tests import cases
+from oracle import quantized_matmul_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+  import xla_amd.experimental.custom_kernel  # noqa: F401  (defines both ops)
+  import xla_amd.experimental.xla_quantized_matmul as qmm
+  return qmm
+
+
+def dev(*ts):
+  return [None if t is None else t.cuda() for t in ts]
+
+
+def check(actual, expected, what=""):
+  assert actual.dtype == expected.dtype, f"{what}: dtype {actual.dtype} vs {expected.dtype}"
+  assert actual.shape == expected.shape
+  a = actual.cpu()
+  assert torch.isfinite(a.float()).all()
+  rl2 = cases.rel_l2(a, expected)
+  assert cases.within_tolerance(a, expected), f"{what}: rel-L2 {rl2:.3e} outside tolerance"
+  return rl2
+
+
+# ---- config 1: fp32 per-channel -------------------------------------------------
+def test_config1_fp32_per_channel(ops):
+  x, w, s = cases.uniform_int8(8, 1024, 1024, torch.float32, torch.float32, seed=1)
+  exp = oracle.quantized_matmul(x, w, s)
+  xd, wd, sd = dev(x, w, s)
+  out = torch.ops.xla.quantized_matmul(xd, wd, sd)
+  rl2 = check(out, exp, "cfg1")
+  assert rl2 < 1e-5  # fp32 path: summation order only
+  assert ops.counters["skinny_mfma"] >= 1
+
+
+# ---- config 2: decode GEMV, bf16 ---------------------------------------------------
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_config2_decode_gemv(ops, m):
+  x, w, s, _ = cases.per_channel_int8(m, 14336, 4096, torch.bfloat16, torch.bfloat16, seed=2)
+  exp = oracle.quantized_matmul(x, w, s)
+  xd, wd, sd = dev(x, w, s)
+  out = torch.ops.xla.quantized_matmul(xd, wd, sd)
+  rl2 = check(out, exp, f"cfg2 M={m}")
+  # two-rounding epilogue reproduced: only summation-order ulp flips remain
+  assert rl2 < 5e-4, rl2
+
+
+@pytest.mark.parametrize("m,n,k", [(3, 50, 128), (17, 100, 256), (33, 16, 384), (70, 31, 128)])
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("zp", [False, True])
+def test_skinny_per_channel_shapes(ops, m, n, k, xdt, zp):
+  x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)
+  z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(xdt) if zp else None
+  exp = oracle.quantized_matmul(x, w, s, z)
+  xd, wd, sd, zd = dev(x, w, s, z)
+  before = ops.counters["skinny_mfma"]
+  out = torch.ops.xla.quantized_matmul(xd, wd, sd, zd)
+  assert ops.counters["skinny_mfma"] == before + 1
+  check(out, exp, "skinny per-channel")
+
+
+def test_per_channel_mixed_scale_dtype(ops):
+  x, w, s, _ = cases.per_channel_int8(5, 64, 256, torch.bfloat16, torch.float32, seed=3)
+  z = torch.randn(64, generator=cases.gen(6)) * 0.01
+  exp = oracle.quantized_matmul(x, w, s, z)
+  out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z))
+  assert out.dtype == torch.float32
+  check(out, exp, "bf16 x, f32 scale/zp")
+
+
+# ---- small odd shapes: generic kernel ----------------------------------------------
+@pytest.mark.parametrize("xdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("zp", [False, True])
+def test_generic_small(ops, xdt, zp):
+  g = cases.gen(7)
+  x = torch.randn(3, 5, generator=g).to(xdt)
+  w = torch.randint(-128, 128, (8, 5), generator=g, dtype=torch.int32).to(torch.int8)
+  s = torch.rand(8, generator=g).to(xdt)
+  z = torch.randn(8, generator=g).to(xdt) if zp else None
+  exp = oracle.quantized_matmul(x, w, s, z)
+  before = ops.counters["generic"]
+  out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z))
+  assert ops.counters["generic"] == before + 1
+  check(out, exp, "generic")
+  # batch dims
+  x3 = torch.randn(2, 3, 5, generator=g).to(xdt)
+  exp = oracle.quantized_matmul(x3, w, s, z)
+  out = torch.ops.xla.quantized_matmul(*dev(x3, w, s, z))
+  check(out, exp, "generic 3-D x")
+
+
+# ---- config 3: blockwise int4 ----------------------------------------------------------
+@pytest.mark.parametrize("bits,int4", [(4, True), (4, False), (8, False)])
+@pytest.mark.parametrize("sym", [False, True])
+def test_config3_blockwise(ops, bits, int4, sym):
+  x, w, s, z, _ = cases.blockwise(16, 4096, 4096, 128, bits, torch.bfloat16, symmetric=sym, seed=4)
+  exp = oracle.quantized_matmul(x, w, s, z, block_size=128)
+  out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=128, int4_weight=int4)
+  rl2 = check(out, exp, "cfg3")
+  assert rl2 < 1e-3, rl2
+
+
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_blockwise_shapes(ops, xdt, bits):
+  for (m, n, k, c) in [(2, 24, 256, 128), (19, 40, 512, 256), (3, 8, 6, 2), (5, 16, 96, 32)]:
+    x, w, s, z, _ = cases.blockwise(m, n, k, c, bits, xdt, symmetric=False, seed=m)
+    exp = oracle.quantized_matmul(x, w, s, z, block_size=c)
+    out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=c, int4_weight=(bits == 4))
+    check(out, exp, f"blockwise {m,n,k,c}")
+
+
+def test_int4_per_channel(ops):
+  g = cases.gen(9)
+  x = torch.randn(7, 512, generator=g).bfloat16()
+  w = torch.randint(-8, 8, (48, 512), generator=g, dtype=torch.int32).to(torch.int8)
+  s = torch.rand(48, generator=g).bfloat16()
+  exp = oracle.quantized_matmul(x, w, s)
+  out = torch.ops.xla.quantized_matmul(*dev(x, w, s), int4_weight=True)
+  check(out, exp, "int4 per-channel")
+
+
+# ---- activation quantizer: bit exact ---------------------------------------------------
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("policy", ["saturate", "wrap"])
+def test_quantize_per_token_bit_exact(ops, xdt, policy):
+  for (m, k) in [(64, 4096), (5, 37), (3, 8), (1, 16384)]:
+    x = cases.outlier_activations(m, k, xdt, seed=11 + m)
+    if m >= 3:
+      x[1] = 0  # all-zero row
+    q_ref, s_ref = oracle.quantize_tensor(x, overflow=policy)
+    q, s, xs = ops.quantize_per_token_gpu(x.cuda(), want_sum=True, overflow=policy)
+    assert torch.equal(q.cpu(), q_ref), f"{xdt} {policy} {(m, k)}: {(q.cpu() != q_ref).sum().item()} mismatches"
+    assert torch.equal(s.cpu(), s_ref)
+    assert torch.equal(xs.cpu().long(), q_ref.long().sum(-1))
+
+
+def test_quantize_all_bf16_values(ops):
+  bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+  vals = bits.view(torch.bfloat16)
+  finite = torch.isfinite(vals.float())
+  vals = vals[finite]
+  rows = []
+  for mx in [1.0, 1.5, 3.140625, 100.0, 2.0**-20, 2.0**60]:
+    v = vals[vals.float().abs() <= mx]
+    row = torch.zeros(65536, dtype=torch.bfloat16)
+    row[:v.numel()] = v
+    row[-1] = mx
+    rows.append(row)
+  x = torch.stack(rows)
+  for policy in ("saturate", "wrap"):
+    q_ref, s_ref = oracle.quantize_tensor(x, overflow=policy)
+    q, s, _ = ops.quantize_per_token_gpu(x.cuda(), overflow=policy)
+    assert torch.equal(q.cpu(), q_ref)
+    assert torch.equal(s.cpu(), s_ref)
+
+
+# ---- W8A8: int32 accumulators bit exact, epilogue within tolerance ------------------------
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (100, 130, 256), (256, 512, 128), (300, 700, 1024),
+                                   (2048, 1024, 512), (7, 9, 80), (5, 8, 5), (512, 4096, 4096)])
+def test_w8a8_int32_exact(ops, m, n, k):
+  g = cases.gen(m + n + k)
+  xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+  w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+  xs = torch.rand(m, 1, generator=g)
+  ws = torch.rand(n, generator=g)
+  _, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), xs.cuda(), ws.cuda(), None, None,
+                             cvt_dtype=torch.float32, mid_dtype=torch.float32,
+                             out_dtype=torch.float32, want_acc=True)
+  ref = torch.from_numpy(xq.numpy().astype(np.int64) @ w.numpy().astype(np.int64).T)
+  assert torch.equal(acc.cpu().long(), ref)
+
+
+@pytest.mark.parametrize("xdt,sdt", [(torch.bfloat16, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                     (torch.float32, torch.float32), (torch.float16, torch.float32)])
+@pytest.mark.parametrize("zp", [False, True])
+def test_w8a8_quantized_matmul(ops, xdt, sdt, zp):
+  m, n, k = 200, 384, 512
+  x = cases.outlier_activations(m, k, xdt, seed=21)
+  _, w, s, _ = cases.per_channel_int8(1, n, k, xdt, sdt, seed=22)
+  z = (torch.randn(n, generator=cases.gen(23)) * 0.01).to(sdt) if zp else None
+  exp = oracle.quantized_matmul(x, w, s, z, quantize_activation=True)
+  out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z), quantize_activation=True)
+  rl2 = check(out, exp, "w8a8")
+  assert rl2 < 1e-6 or xdt != torch.float32, rl2
+
+
+def test_config4_w8a8_prefill(ops):
+  m, n, k = 2048, 14336, 4096
+  x = cases.outlier_activations(m, k, torch.bfloat16, seed=1234)
+  _, w, s, _ = cases.per_channel_int8(1, n, k, torch.bfloat16, torch.float32, seed=31)
+  xd, wd, sd = dev(x, w, s)
+  out = torch.ops.xla.quantized_matmul(xd, wd, sd, quantize_activation=True)
+  assert out.dtype == torch.float32 and out.shape == (m, n)
+  # exact int32 accumulators on a sample of rows/columns + the row-checksum identity
+  xq_ref, xs_ref = oracle.quantize_tensor(x)
+  xq, xs, _ = ops.quantize_per_token_gpu(xd)
+  assert torch.equal(xq.cpu(), xq_ref) and torch.equal(xs.cpu(), xs_ref)
+  _, acc = ops.w8a8_gemm_gpu(xq, wd, xs, sd, None, None, cvt_dtype=torch.float32,
+                             mid_dtype=torch.float32, out_dtype=torch.float32, want_acc=True)
+  acc = acc.cpu()
+  rows = torch.arange(0, m, 37)
+  ref_rows = oracle.int32_accumulators(xq_ref[rows], w)
+  assert torch.equal(acc[rows], ref_rows)
+  cols = torch.arange(0, n, 101)
+  ref_cols = oracle.int32_accumulators(xq_ref, w[cols])
+  assert torch.equal(acc[:, cols], ref_cols)
+  # checksum: sum_n acc[m,n] == x_q[m,:] . sum_n w[n,:]
+  wsum = w.long().sum(0)
+  assert torch.equal(acc.long().sum(1), xq_ref.long() @ wsum)
+  exp_rows = oracle.quantized_matmul(x[rows], w, s, quantize_activation=True)
+  check(out[rows.cuda()], exp_rows, "cfg4 rows")
+
+
+def test_quantized_matmul_int8_op(ops):
+  for (m, n, k, hit) in [(256, 4096, 4096, True), (192, 320, 256, False)]:
+    x = cases.outlier_activations(m, k, torch.bfloat16, seed=41)
+    _, w, s, _ = cases.per_channel_int8(1, n, k, torch.bfloat16, torch.float32, seed=42)
+    exp = oracle.quantized_matmul_int8(x, w, s, quantize_activation=True) if hit else \
+        oracle.quantized_matmul_int8_fallback(x, w, s, quantize_activation=True)
+    out = torch.ops.xla.quantized_matmul_int8(*dev(x, w, s), quantize_activation=True)
+    assert out.dtype == torch.bfloat16
+    check(out, exp, "quantized_matmul_int8")

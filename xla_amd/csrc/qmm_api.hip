@@ -1,0 +1,51 @@
+// Error reporting, version and the shape-based dispatcher of libxla_amd_qmm.so.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "qmm_common.h"
+
+static thread_local char g_err[512] = "";
+
+int qmm_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int qmm_check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return XLA_AMD_QMM_OK;
+  return qmm_fail(XLA_AMD_QMM_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+extern "C" int xla_amd_qmm_abi_version(void) { return XLA_AMD_QMM_ABI_VERSION; }
+
+extern "C" const char* xla_amd_qmm_last_error(void) { return g_err; }
+
+extern "C" size_t xla_amd_qmm_packed_bytes(int64_t N, int64_t K, int bits) {
+  if (N <= 0 || K <= 0) return 0;
+  if (bits == 8) return (size_t)N * (size_t)K;
+  if (bits == 4 && K % 8 == 0) return (size_t)N * (size_t)K / 2;
+  return 0;
+}
+
+// The two regimes of a quantized linear layer on MI355X:
+//  * few rows of x (decode): every weight byte is used M times, far below the
+//    ~630 int8 ops/byte (or ~310 bf16 flops/byte) the chip can do per HBM
+//    byte, so the weight is streamed exactly once by the skinny kernel;
+//  * many rows with int8 activations (prefill): LDS-tiled int8 MFMA GEMM.
+// Shapes neither fast kernel accepts run the one-thread-per-output kernels.
+extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, int bits,
+                                    int x_dt, int quantize_activation) {
+  (void)N;
+  (void)x_dt;
+  if (quantize_activation) {
+    if (K % 64 == 0 && M * N >= 64 * 64) return XLA_AMD_KERNEL_W8A8_MFMA;
+    return XLA_AMD_KERNEL_W8A8_GENERIC;
+  }
+  if (C <= 0) C = K;
+  if (K % 128 == 0 && C % 128 == 0 && (bits == 8 || bits == 4) && M >= 1)
+    return XLA_AMD_KERNEL_SKINNY_MFMA;
+  return XLA_AMD_KERNEL_GENERIC;
+}

@@ -1,0 +1,78 @@
+// Shared host/device helpers of libxla_amd_qmm.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "xla_amd_qmm.h"
+
+// ---- host side -------------------------------------------------------------
+// printf-style setter of the calling thread's error text; returns `code`.
+int qmm_fail(int code, const char* fmt, ...);
+// Maps a HIP status to XLA_AMD_QMM_OK / XLA_AMD_QMM_EHIP (recording the text).
+int qmm_check_hip(hipError_t e, const char* what);
+// Error of the launch that was just issued on the calling thread.
+#define QMM_CHECK_LAUNCH(what) qmm_check_hip(hipGetLastError(), what)
+
+static inline bool qmm_valid_dt(int dt) { return dt >= XLA_AMD_DT_F32 && dt <= XLA_AMD_DT_F16; }
+static inline int qmm_dt_size(int dt) { return dt == XLA_AMD_DT_F32 ? 4 : 2; }
+// torch's type promotion between two floating dtypes: equal -> itself,
+// anything else involving f32, or bf16 with f16 -> f32.
+__host__ __device__ static inline int qmm_promote(int a, int b) { return a == b ? a : XLA_AMD_DT_F32; }
+
+// ---- device side -----------------------------------------------------------
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ float qmm_bf16_to_f32(uint16_t b) {
+  return __uint_as_float(((uint32_t)b) << 16);
+}
+
+// Round-to-nearest-even f32 -> bf16 bit pattern (NaN stays NaN).
+__device__ __forceinline__ uint16_t qmm_f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ float qmm_f16_to_f32(uint16_t h) {
+  _Float16 v;
+  __builtin_memcpy(&v, &h, 2);
+  return (float)v;
+}
+
+__device__ __forceinline__ uint16_t qmm_f32_to_f16(float f) {
+  _Float16 v = (_Float16)f;  // v_cvt_f16_f32: round-to-nearest-even
+  uint16_t h;
+  __builtin_memcpy(&h, &v, 2);
+  return h;
+}
+
+// Value of f after a round trip through dtype dt (what storing a torch tensor
+// of that dtype and reading it back does).
+__device__ __forceinline__ float qmm_round_dt(float f, int dt) {
+  if (dt == XLA_AMD_DT_BF16) return qmm_bf16_to_f32(qmm_f32_to_bf16(f));
+  if (dt == XLA_AMD_DT_F16) return qmm_f16_to_f32(qmm_f32_to_f16(f));
+  return f;
+}
+
+__device__ __forceinline__ float qmm_load(const void* p, int64_t i, int dt) {
+  if (dt == XLA_AMD_DT_BF16) return qmm_bf16_to_f32(((const uint16_t*)p)[i]);
+  if (dt == XLA_AMD_DT_F16) return qmm_f16_to_f32(((const uint16_t*)p)[i]);
+  return ((const float*)p)[i];
+}
+
+// Stores a value that is already on dt's grid (or rounds it there).
+__device__ __forceinline__ void qmm_store(void* p, int64_t i, float v, int dt) {
+  if (dt == XLA_AMD_DT_BF16)
+    ((uint16_t*)p)[i] = qmm_f32_to_bf16(v);
+  else if (dt == XLA_AMD_DT_F16)
+    ((uint16_t*)p)[i] = qmm_f32_to_f16(v);
+  else
+    ((float*)p)[i] = v;
+}

@@ -1,0 +1,160 @@
+// Per-token dynamic int8 quantization of activations (HBM-bound elementwise +
+// row reduction).  One workgroup per row; the row is read twice (the second
+// read hits L2: a row is at most a few tens of KB), so x is streamed from HBM
+// once and x_q written once.
+//
+// The arithmetic is the reference's, op by op, in x's dtype:
+//   max = amax(|x|); scale = RN_x(max / 127); r = RN_x(x / scale); q = int8(rint(r))
+// RN_x(a / b) is obtained as RN_x(RN_f32(a / b)): a and b carry at most 11
+// significant bits, so the f32 quotient never straddles a rounding boundary of
+// the narrower type unless it is exact.
+#include "qmm_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_sum(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ int quantize_one(float xv, float scale, int x_dt, int policy) {
+  float r = rintf(qmm_round_dt(xv / scale, x_dt));  // rintf: round half to even
+  if (!(fabsf(r) <= 3.0e38f)) r = 0.f;              // NaN/inf (zero scale) -> 0
+  if (policy == XLA_AMD_OVERFLOW_SATURATE) return (int)fminf(fmaxf(r, -128.f), 127.f);
+  r = fminf(fmaxf(r, -2147483648.f), 2147483520.f);
+  return (int)(int8_t)(int)r;
+}
+
+// VEC = elements per thread per step: 8 (16-byte loads of 2-byte types, two
+// for f32) when K % 8 == 0 and the row starts are 16-byte aligned, else 1.
+template <int XT, int VEC>
+__global__ void __launch_bounds__(kThreads)
+qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* __restrict__ x_scale,
+                    int32_t* __restrict__ x_sum, int64_t K, int scale_out_dt, int policy) {
+  __shared__ float smax[kThreads / 64];
+  __shared__ int ssum[kThreads / 64];
+  const int64_t m = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  constexpr int esz = XT == XLA_AMD_DT_F32 ? 4 : 2;
+  const char* xrow = (const char*)x + (size_t)m * K * esz;
+
+  auto load_vec = [&](int64_t k, float* f) {
+    if constexpr (VEC == 1) {
+      f[0] = qmm_load(xrow, k, XT);
+    } else if constexpr (XT == XLA_AMD_DT_F32) {
+      const f32x4* p = (const f32x4*)(xrow + k * 4);
+      f32x4 a = p[0], b = p[1];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { f[i] = a[i]; f[4 + i] = b[i]; }
+    } else {
+      i32x4 a = *(const i32x4*)(xrow + k * 2);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        uint32_t d = (uint32_t)a[i];
+        if constexpr (XT == XLA_AMD_DT_BF16) {
+          f[2 * i] = __uint_as_float(d << 16);
+          f[2 * i + 1] = __uint_as_float(d & 0xffff0000u);
+        } else {
+          f[2 * i] = qmm_f16_to_f32((uint16_t)(d & 0xffffu));
+          f[2 * i + 1] = qmm_f16_to_f32((uint16_t)(d >> 16));
+        }
+      }
+    }
+  };
+
+  // pass 1: row abs-max
+  float mx = 0.f;
+  for (int64_t k = (int64_t)tid * VEC; k < K; k += (int64_t)kThreads * VEC) {
+    float f[VEC];
+    load_vec(k, f);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      float av = fabsf(f[i]);
+      mx = (av > mx || av != av) ? av : mx;  // propagate NaN like torch.amax
+    }
+  }
+  mx = wave_max(mx);
+  if (lane == 0) smax[wv] = mx;
+  __syncthreads();
+  mx = smax[0];
+#pragma unroll
+  for (int i = 1; i < kThreads / 64; ++i) mx = fmaxf(mx, smax[i]);
+  const float scale = qmm_round_dt(mx / 127.0f, XT);
+
+  // pass 2: quantize
+  int lsum = 0;
+  for (int64_t k = (int64_t)tid * VEC; k < K; k += (int64_t)kThreads * VEC) {
+    float f[VEC];
+    load_vec(k, f);
+    int q[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      q[i] = quantize_one(f[i], scale, XT, policy);
+      lsum += q[i];
+    }
+    if constexpr (VEC == 1) {
+      xq[(size_t)m * K + k] = (int8_t)q[0];
+    } else {
+      uint32_t lo = 0, hi = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        lo |= ((uint32_t)(uint8_t)q[i]) << (8 * i);
+        hi |= ((uint32_t)(uint8_t)q[4 + i]) << (8 * i);
+      }
+      i32x2 v = {(int)lo, (int)hi};
+      *(i32x2*)(xq + (size_t)m * K + k) = v;
+    }
+  }
+  if (tid == 0) qmm_store(x_scale, m, scale, scale_out_dt);
+  if (x_sum) {
+    lsum = wave_sum(lsum);
+    if (lane == 0) ssum[wv] = lsum;
+    __syncthreads();
+    if (tid == 0) {
+      int t = 0;
+#pragma unroll
+      for (int i = 0; i < kThreads / 64; ++i) t += ssum[i];
+      x_sum[m] = t;
+    }
+  }
+}
+
+template <int XT>
+int launch(const void* x, int8_t* xq, void* x_scale, int32_t* x_sum, int64_t M, int64_t K,
+           int scale_out_dt, int policy, bool vec, hipStream_t stream) {
+  if (vec)
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8>), dim3((unsigned)M), dim3(kThreads), 0, stream, x,
+                       xq, x_scale, x_sum, K, scale_out_dt, policy);
+  else
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 1>), dim3((unsigned)M), dim3(kThreads), 0, stream, x,
+                       xq, x_scale, x_sum, K, scale_out_dt, policy);
+  return QMM_CHECK_LAUNCH("quantize_per_token launch");
+}
+
+}  // namespace
+
+extern "C" int xla_amd_qmm_quantize_per_token(const void* x, int8_t* x_q, void* x_scale,
+                                              int32_t* x_sum, int64_t M, int64_t K, int x_dt,
+                                              int scale_out_dt, int overflow_policy, void* stream) {
+  if (!x || !x_q || !x_scale) return qmm_fail(XLA_AMD_QMM_EINVAL, "quantize_per_token: null pointer");
+  if (M < 0 || K <= 0 || M > 0x7fffffffLL)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "quantize_per_token: bad sizes M=%lld K=%lld", (long long)M, (long long)K);
+  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_out_dt))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "quantize_per_token: bad dtype enum");
+  if (overflow_policy != XLA_AMD_OVERFLOW_SATURATE && overflow_policy != XLA_AMD_OVERFLOW_WRAP)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "quantize_per_token: bad overflow policy %d", overflow_policy);
+  if (M == 0) return XLA_AMD_QMM_OK;
+  bool vec = (K % 8 == 0) && (((uintptr_t)x & 15) == 0) && (((uintptr_t)x_q & 7) == 0);
+  hipStream_t s = (hipStream_t)stream;
+  if (x_dt == XLA_AMD_DT_BF16) return launch<XLA_AMD_DT_BF16>(x, x_q, x_scale, x_sum, M, K, scale_out_dt, overflow_policy, vec, s);
+  if (x_dt == XLA_AMD_DT_F16) return launch<XLA_AMD_DT_F16>(x, x_q, x_scale, x_sum, M, K, scale_out_dt, overflow_policy, vec, s);
+  return launch<XLA_AMD_DT_F32>(x, x_q, x_scale, x_sum, M, K, scale_out_dt, overflow_policy, vec, s);
+}

@@ -1,0 +1,268 @@
+// W8A8 GEMM for gfx950: out[m,n] = epilogue( sum_k x_q[m,k] * w[n,k] ), int8
+// operands, int32 accumulation on the matrix cores (v_mfma_i32_32x32x32_i8),
+// both operands K-contiguous, tiles staged through LDS with a two-stage
+// pipeline, scale epilogue fused.
+//
+// Tiling.  A workgroup of WM x WN waves owns a BM x BN tile of the output and
+// walks K in steps of kBK = 128 bytes.  Each wave owns (BM/WM) x (BN/WN)
+// outputs as a grid of 32x32 MFMA tiles whose int32 accumulators never leave
+// registers.  LDS holds, per stage, the A tile [BM][128] and the B tile
+// [BN][128] as 16-byte chunks with an XOR swizzle (chunk ^= (row/2) % 8) so
+// that the 16 rows x 16 bytes read by a quarter wave for an MFMA operand land
+// in 64 distinct banks, and so do the 2 rows x 8 chunks a quarter wave writes.
+//
+// MFMA operand/result mapping (A = x_q rows, B = w rows):
+//   operand: lane l supplies row l%32, 16 bytes of k at chunk l/32 of a 32-byte step
+//   result : acc[v] of lane l is D[8*(v/4) + 4*(l/32) + v%4][l%32]  (row = m, col = n)
+// so one result register of a wave is 32 consecutive n of a row: coalesced stores.
+#include "qmm_common.h"
+
+int qmm_w8a8_generic_launch(const int8_t* xq, const int8_t* w, const void* x_scale,
+                            const void* w_scale, const void* zp, const int32_t* x_sum, void* out,
+                            int32_t* acc_out, int64_t M, int64_t N, int64_t K, int x_scale_dt,
+                            int w_scale_dt, int zp_dt, int cvt_dt, int mid_dt, int zpo_dt,
+                            int out_dt, hipStream_t stream);
+
+namespace {
+
+constexpr int kBK = 128;  // bytes (= int8 elements) of K per pipeline stage
+
+struct GemmArgs {
+  const int8_t* a;  // x_q [M,K]
+  const int8_t* b;  // w   [N,K]
+  const void* x_scale;
+  const void* w_scale;
+  const void* zp;
+  const int32_t* x_sum;
+  void* out;
+  int32_t* acc_out;
+  int M, N, K;
+  int x_scale_dt, w_scale_dt, zp_dt, cvt_dt, mid_dt, zpo_dt, out_dt;
+  int tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
+
+template <int BM, int BN, int WM, int WN>
+__global__ void __launch_bounds__(WM * WN * 64)
+qmm_w8a8_gemm_kernel(GemmArgs g) {
+  constexpr int T = WM * WN * 64;
+  constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
+  constexpr int MI = TM / 32, NI = TN / 32;  // 32x32 MFMA tiles per wave
+  constexpr int A_CH = BM * 8 / T, B_CH = BN * 8 / T;  // 16-byte chunks per thread per stage
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be a multiple of 32");
+  static_assert((BM * 8) % T == 0 && (BN * 8) % T == 0, "tile rows must divide over the threads");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* sA = smem;                      // [2][BM][128]
+  char* sB = smem + 2 * BM * kBK;       // [2][BN][128]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  // Workgroup -> tile.  Consecutive workgroup ids go to different XCDs (8 of
+  // them, each with its own L2), so give every XCD a contiguous run of tiles
+  // and walk a run down M first: the workgroups an XCD runs together then
+  // share a few B (weight) panels and all A panels through its L2.
+  int bid = blockIdx.x;
+  const int ntiles = g.tiles_m * g.tiles_n;
+  {
+    const int per = (ntiles + 7) / 8;
+    const int xcd = bid & 7, loc = bid >> 3;
+    bid = xcd * per + loc;  // the grid has 8 * per workgroups; the excess ones have no tile
+  }
+  if (bid >= ntiles) return;
+  const int tile_m = bid % g.tiles_m, tile_n = bid / g.tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int K = g.K;
+
+  // Global source of this thread's chunks (row clamped into the matrix).
+  const int8_t* ga[A_CH];
+  const int8_t* gb[B_CH];
+  int lds_a[A_CH], lds_b[B_CH];
+  const int ck = tid & 7;  // chunk within the 128-byte row segment
+#pragma unroll
+  for (int i = 0; i < A_CH; ++i) {
+    int row = (i * T + tid) >> 3;
+    ga[i] = g.a + (size_t)min(m0 + row, g.M - 1) * K + ck * 16;
+    lds_a[i] = row * kBK + swz(row, ck) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < B_CH; ++i) {
+    int row = (i * T + tid) >> 3;
+    gb[i] = g.b + (size_t)min(n0 + row, g.N - 1) * K + ck * 16;
+    lds_b[i] = row * kBK + swz(row, ck) * 16;
+  }
+
+  i32x4 ra[A_CH], rb[B_CH];
+  auto gload = [&](int k0) {
+    const bool in = (k0 + ck * 16) < K;  // K tail: chunks past K read as zero
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) ra[i] = in ? *(const i32x4*)(ga[i] + k0) : i32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) rb[i] = in ? *(const i32x4*)(gb[i] + k0) : i32x4{0, 0, 0, 0};
+  };
+  auto sstore = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) *(i32x4*)(sA + stage * BM * kBK + lds_a[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) *(i32x4*)(sB + stage * BN * kBK + lds_b[i]) = rb[i];
+  };
+
+  i32x16 acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+
+  const int lrow = lane & 31, lchunk = lane >> 5;
+  auto compute = [&](int stage) {
+    const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
+    const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
+#pragma unroll
+    for (int ks = 0; ks < kBK / 32; ++ks) {
+      i32x4 af[MI], bf[NI];
+      const int c = 2 * ks + lchunk;
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        int row = i * 32 + lrow;
+        af[i] = *(const i32x4*)(a_base + row * kBK + swz(wm * TM + row, c) * 16);
+      }
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        int row = j * 32 + lrow;
+        bf[j] = *(const i32x4*)(b_base + row * kBK + swz(wn * TN + row, c) * 16);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  const int ksteps = (K + kBK - 1) / kBK;
+  gload(0);
+  sstore(0);
+  __syncthreads();
+  for (int kt = 0; kt < ksteps; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < ksteps) gload((kt + 1) * kBK);
+    compute(cur);
+    if (kt + 1 < ksteps) sstore(cur ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue.
+  const bool has_zp = g.zp != nullptr;
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int n = n0 + wn * TN + j * 32 + lrow;
+    const bool n_ok = n < g.N;
+    float ws = 0.f, zpv = 0.f;
+    if (g.out && n_ok) {
+      ws = qmm_load(g.w_scale, n, g.w_scale_dt);
+      if (has_zp) zpv = qmm_load(g.zp, n, g.zp_dt);
+    }
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int m = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * lchunk + (v & 3);
+        if (!n_ok || m >= g.M) continue;
+        const int a = acc[i][j][v];
+        const size_t idx = (size_t)m * g.N + n;
+        if (g.acc_out) g.acc_out[idx] = a;
+        if (g.out) {
+          float val = qmm_round_dt((float)a, g.cvt_dt);
+          val = qmm_round_dt(val * ws, g.mid_dt);
+          if (has_zp) {
+            float z = qmm_round_dt(qmm_round_dt((float)g.x_sum[m], g.zpo_dt) * zpv, g.zpo_dt);
+            val = qmm_round_dt(val - z, g.mid_dt);
+          }
+          val = qmm_round_dt(val * qmm_load(g.x_scale, m, g.x_scale_dt), g.out_dt);
+          qmm_store(g.out, idx, val, g.out_dt);
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_tile(GemmArgs g, hipStream_t stream) {
+  g.tiles_m = (g.M + BM - 1) / BM;
+  g.tiles_n = (g.N + BN - 1) / BN;
+  const int ntiles = g.tiles_m * g.tiles_n;
+  const int per = (ntiles + 7) / 8;
+  const unsigned grid = (unsigned)(per * 8);
+  constexpr size_t lds = 2 * (size_t)(BM + BN) * kBK;
+  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN>;
+  static thread_local bool attr_set = false;
+  if (!attr_set) {
+    int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
+                           "w8a8_gemm hipFuncSetAttribute");
+    if (rc != XLA_AMD_QMM_OK) return rc;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, stream, g);
+  return QMM_CHECK_LAUNCH("w8a8_gemm launch");
+}
+
+}  // namespace
+
+// Tile choice by shape: big tiles when the grid still fills 256 CUs, smaller
+// ones for small problems.
+static void choose_tile(int64_t M, int64_t N, int* bm, int* bn) {
+  auto tiles = [&](int a, int b) { return ((M + a - 1) / a) * ((N + b - 1) / b); };
+  if (M > 128 && N > 128 && tiles(256, 256) >= 200) { *bm = 256; *bn = 256; return; }
+  if (M > 64 && tiles(128, 128) >= 128) { *bm = 128; *bn = 128; return; }
+  *bm = 64; *bn = 64;
+}
+
+extern "C" int xla_amd_qmm_w8a8_tile(int64_t M, int64_t N, int64_t K, int32_t* tile_mnk) {
+  if (!tile_mnk || M <= 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_tile: bad arguments");
+  int bm, bn;
+  choose_tile(M, N, &bm, &bn);
+  tile_mnk[0] = bm; tile_mnk[1] = bn; tile_mnk[2] = kBK;
+  return XLA_AMD_QMM_OK;
+}
+
+extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const void* x_scale,
+                                     const void* w_scale, const void* zp, const int32_t* x_sum,
+                                     void* out, int32_t* acc_out, int64_t M, int64_t N, int64_t K,
+                                     int x_scale_dt, int w_scale_dt, int zp_dt, int cvt_dt,
+                                     int mid_dt, int zpo_dt, int out_dt, int block_m, int block_n,
+                                     void* stream) {
+  if (!x_q || !w) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_gemm: null operand");
+  if (!out && !acc_out) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_gemm: neither out nor acc_out given");
+  if (out && (!x_scale || !w_scale)) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_gemm: null scale");
+  if ((zp != nullptr) != (x_sum != nullptr) && out)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_gemm: zp and x_sum must be given together");
+  if (M < 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_gemm: bad sizes");
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_gemm: dimension too large");
+  if (out && (!qmm_valid_dt(x_scale_dt) || !qmm_valid_dt(w_scale_dt) || !qmm_valid_dt(cvt_dt) ||
+              !qmm_valid_dt(mid_dt) || !qmm_valid_dt(out_dt) ||
+              (zp && (!qmm_valid_dt(zp_dt) || !qmm_valid_dt(zpo_dt)))))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_gemm: bad dtype enum");
+  if (M == 0) return XLA_AMD_QMM_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool fast = (K % 16 == 0) && ((((uintptr_t)x_q | (uintptr_t)w) & 15) == 0);
+  if (!fast)
+    return qmm_w8a8_generic_launch(x_q, w, x_scale, w_scale, zp, x_sum, out, acc_out, M, N, K,
+                                   x_scale_dt, w_scale_dt, zp_dt, cvt_dt, mid_dt, zpo_dt, out_dt, s);
+  GemmArgs g;
+  g.a = x_q; g.b = w; g.x_scale = x_scale; g.w_scale = w_scale; g.zp = out ? zp : nullptr;
+  g.x_sum = x_sum; g.out = out; g.acc_out = acc_out;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.x_scale_dt = x_scale_dt; g.w_scale_dt = w_scale_dt; g.zp_dt = zp_dt; g.cvt_dt = cvt_dt;
+  g.mid_dt = mid_dt; g.zpo_dt = zpo_dt; g.out_dt = out_dt;
+  g.tiles_m = g.tiles_n = 0;
+  int bm = block_m, bn = block_n;
+  if (bm == 0 && bn == 0) choose_tile(M, N, &bm, &bn);
+  if (bm == 256 && bn == 256) return launch_tile<256, 256, 2, 2>(g, s);
+  if (bm == 128 && bn == 128) return launch_tile<128, 128, 2, 2>(g, s);
+  if (bm == 64 && bn == 64) return launch_tile<64, 64, 2, 2>(g, s);
+  return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_gemm: no kernel for tile %dx%d", bm, bn);
+}
