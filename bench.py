@@ -1,0 +1,253 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+A "step" is one call of torch.ops.xla.quantized_matmul on the decode-GEMV
+configuration (x bf16 [16,4096], w int8 [14336,4096], scaler bf16 [14336]),
+with every input already resident in HBM.  The weight rotates over enough
+distinct copies (> 512 MB) that neither L2 nor the 256 MB Infinity Cache can
+hold it, so the reported bandwidth is HBM bandwidth.  The K timed steps are
+captured once into a HIP graph and replayed (a decode step is launch-bound
+otherwise); `--no-graph` times eager calls instead.
+
+Prints ONE JSON line.  `value` is algorithmic GB/s of the whole timed region
+(wall clock between device synchronisations); `roofline` is the same kernel
+measured with HIP events on its stream; `cpu_baseline` is the CPU oracle timed
+on this host; `extra` carries the other configurations (M=1/4, hot cache,
+blockwise int4, W8A8 prefill GEMM with its own MFMA roofline, the 7 linears of
+a Llama-3-8B layer).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA (5.0 POP/s)
+
+N_OUT, K_IN = 14336, 4096
+
+
+def gemv_bytes(m, n, k, w_bytes_per_elem=1.0, x_b=2, s_b=2, out_b=2, n_scale_rows=1, zp=False):
+  """Algorithmic bytes: weight + activations + scale(+zp) + output."""
+  scale_bytes = n * s_b * n_scale_rows * (2 if zp else 1)
+  return int(n * k * w_bytes_per_elem + m * k * x_b + scale_bytes + m * n * out_b)
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=240)
+  ap.add_argument("--warmup", type=int, default=48)
+  ap.add_argument("--no-graph", action="store_true", help="time eager calls instead of a HIP graph replay")
+  ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    print("bench.py: this build measures one GPU; --gpus must be 1 (the kernels are not sharded, "
+          "see DESIGN.md for how the path would shard)", file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+  if not torch.cuda.is_available():
+    print("bench.py: no GPU visible", file=sys.stderr)
+    sys.exit(3)
+  from xla_amd import _lib
+  _lib.load()  # no fallback: fail here if the HIP library is missing
+  import xla_amd.experimental.custom_kernel  # noqa: F401
+  import xla_amd.experimental.xla_quantized_matmul as qmm
+  from tests import cases
+
+  dev = torch.device("cuda:0")
+  torch.cuda.set_device(dev)
+  op = torch.ops.xla.quantized_matmul
+
+  def time_calls(fns, steps, warmup, graph=True):
+    """fns: list of zero-arg callables used round-robin.  Returns (wall_ms_per_step, event_ms_per_step)."""
+    for i in range(warmup):
+      fns[i % len(fns)]()
+    torch.cuda.synchronize()
+    g = None
+    if graph:
+      try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+          for i in range(steps):
+            fns[i % len(fns)]()
+        g.replay()  # untimed: first replay uploads the graph
+        torch.cuda.synchronize()
+      except Exception as e:  # capture unsupported for some reason: time eager calls
+        print(f"bench.py: graph capture failed ({e}); timing eager calls", file=sys.stderr)
+        g = None
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    if g is not None:
+      g.replay()
+    else:
+      for i in range(steps):
+        fns[i % len(fns)]()
+    e1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps, g is not None
+
+  use_graph = not args.no_graph
+
+  # ---- headline: decode GEMV, M = 16, rotating (cold) weights -----------------
+  x16, w_cpu, s_cpu, _ = cases.per_channel_int8(16, N_OUT, K_IN, torch.bfloat16, torch.bfloat16, seed=2)
+  n_rot = 12  # 12 x 58.7 MB = 704 MB > 512 MB
+  w0 = w_cpu.to(dev)
+  ws = [w0] + [w0.clone() for _ in range(n_rot - 1)]
+  s_d = s_cpu.to(dev)
+  xs = {m: x16[:m].contiguous().to(dev) for m in (1, 4, 16)}
+
+  def gemv_fns(m, weights):
+    return [(lambda w=w: op(xs[m], w, s_d)) for w in weights]
+
+  wall_ms, ev_ms, graphed = time_calls(gemv_fns(16, ws), args.steps, args.warmup, use_graph)
+  bytes16 = gemv_bytes(16, N_OUT, K_IN)
+  value = bytes16 / (wall_ms * 1e-3) / 1e9
+  achieved = bytes16 / (ev_ms * 1e-3) / 1e9
+
+  result = {
+      "metric": "quantized_matmul HBM GB/s & TOPS (% roofline): int8 decode GEMV + W8A8 GEMM",
+      "value": round(value, 1),
+      "unit": "GB/s",
+      "n_gpus": 1,
+      "steps": args.steps,
+      "warmup": args.warmup,
+      "ms_per_step": round(wall_ms, 6),
+      "higher_is_better": True,
+      "scaling": "weak",
+      "vs_baseline": None,
+      "dtype": "bf16 x int8 -> f32 accumulate -> bf16",
+      "data": "synthetic",
+      "config": {
+          "workload": "decode GEMV, per-channel int8 weight-only: x bf16 [16,4096], w int8 [14336,4096], scaler bf16 [14336]",
+          "weights": f"{n_rot} rotating copies (cold: > Infinity Cache)",
+          "launch": "HIP graph replay" if graphed else "eager calls",
+          "algorithmic_bytes_per_step": bytes16,
+      },
+      "roofline": {
+          "bound": "hbm",
+          "achieved": round(achieved, 1),
+          "peak": HBM_PEAK_GBPS,
+          "unit": "GB/s",
+          "frac": round(achieved / HBM_PEAK_GBPS, 4),
+          "traffic": None,
+          "kernel": "qmm_skinny_kernel<bf16, int8, MT=1>",
+          "avg_launch_us": round(ev_ms * 1e3, 3),
+      },
+  }
+
+  extra = {}
+  if not args.no_extra:
+    steps2 = max(24, args.steps // 2)
+    # decode GEMV at M = 1, 4 (cold) and M = 16 hot (single weight buffer: cache resident)
+    for m in (1, 4):
+      _, ev, _ = time_calls(gemv_fns(m, ws), steps2, 12, use_graph)
+      b = gemv_bytes(m, N_OUT, K_IN)
+      extra[f"gemv_M{m}_cold"] = {"us": round(ev * 1e3, 3), "GBps": round(b / ev / 1e6, 1),
+                                  "frac_hbm": round(b / ev / 1e6 / HBM_PEAK_GBPS, 4)}
+    _, ev, _ = time_calls(gemv_fns(16, ws[:1]), steps2, 12, use_graph)
+    extra["gemv_M16_hot"] = {"us": round(ev * 1e3, 3), "GBps": round(bytes16 / ev / 1e6, 1),
+                             "note": "one weight buffer, served from Infinity Cache; not HBM bandwidth"}
+    del ws[1:]
+
+    # blockwise int4 (config 3)
+    x3, w3, s3, z3, _ = cases.blockwise(16, 4096, 4096, 128, 4, torch.bfloat16, symmetric=False, seed=4)
+    x3d, s3d, z3d = x3.to(dev), s3.to(dev), z3.to(dev)
+    w3s = [w3.to(dev) for _ in range(40)]  # packed copies: 40 x 8.4 MB
+    fns = [(lambda w=w: op(x3d, w, s3d, z3d, block_size=128, int4_weight=True)) for w in w3s]
+    _, ev, _ = time_calls(fns, steps2, 80, use_graph)
+    b3 = gemv_bytes(16, 4096, 4096, 0.5, n_scale_rows=32, zp=True)
+    extra["blockwise_int4_M16"] = {"us": round(ev * 1e3, 3), "GBps": round(b3 / ev / 1e6, 1),
+                                   "frac_hbm": round(b3 / ev / 1e6 / HBM_PEAK_GBPS, 4),
+                                   "algorithmic_bytes": b3}
+    del w3s, fns
+
+    # W8A8 prefill GEMM (config 4)
+    m4 = 2048
+    x4 = cases.outlier_activations(m4, K_IN, torch.bfloat16, seed=1234).to(dev)
+    s4 = s_cpu.float().to(dev)
+    xq, xsc, _ = qmm.quantize_per_token_gpu(x4)
+    steps4 = 20
+    _, ev_q, _ = time_calls([lambda: qmm.quantize_per_token_gpu(x4)], steps4, 5, use_graph)
+    _, ev_g, _ = time_calls([lambda: qmm.w8a8_gemm_gpu(xq, w0, xsc, s4, None, None, cvt_dtype=torch.float32,
+                                                       mid_dtype=torch.float32, out_dtype=torch.float32)],
+                            steps4, 5, use_graph)
+    _, ev_gb, _ = time_calls([lambda: qmm.w8a8_gemm_gpu(xq, w0, xsc, s4, None, None, cvt_dtype=torch.float32,
+                                                        mid_dtype=torch.float32, out_dtype=torch.bfloat16)],
+                             steps4, 5, use_graph)
+    _, ev_e2e, _ = time_calls([lambda: op(x4, w0, s4, quantize_activation=True)], steps4, 5, use_graph)
+    ops4 = 2.0 * m4 * N_OUT * K_IN
+    extra["w8a8_prefill_M2048"] = {
+        "gemm_us_f32_out": round(ev_g * 1e3, 2),
+        "gemm_us_bf16_out": round(ev_gb * 1e3, 2),
+        "quantize_us": round(ev_q * 1e3, 2),
+        "end_to_end_us": round(ev_e2e * 1e3, 2),
+        "roofline": {"bound": "mfma", "achieved": round(ops4 / ev_gb / 1e9, 1), "peak": INT8_PEAK_TOPS,
+                     "unit": "TOP/s", "frac": round(ops4 / ev_gb / 1e9 / INT8_PEAK_TOPS, 4),
+                     "traffic": None, "kernel": "qmm_w8a8_gemm_kernel (bf16 out)"},
+        "tops_f32_out": round(ops4 / ev_g / 1e9, 1),
+        "tops_end_to_end": round(ops4 / ev_e2e / 1e9, 1),
+    }
+    del x4, xq, xsc
+
+    # Llama-3-8B decoder layer, 7 linears (config 5)
+    shapes = {"q": (4096, 4096), "k": (1024, 4096), "v": (1024, 4096), "o": (4096, 4096),
+              "gate": (14336, 4096), "up": (14336, 4096), "down": (4096, 14336)}
+    g5 = cases.gen(5)
+    layer = {}
+    for name, (n, k) in shapes.items():
+      w = torch.randint(-127, 128, (n, k), generator=g5, dtype=torch.int32).to(torch.int8).to(dev)
+      layer[name] = (w, (torch.rand(n, generator=g5) * 0.01).to(dev))
+    for tag, m, qa in (("decode_M32", 32, False), ("prefill_M512", 512, True)):
+      x_in = {4096: torch.randn(m, 4096, generator=g5).bfloat16().to(dev),
+              14336: torch.randn(m, 14336, generator=g5).bfloat16().to(dev)}
+
+      layer_s = {k_: (v[0], v[1] if qa else v[1].bfloat16()) for k_, v in layer.items()}
+
+      def run_layer():
+        for name, (w, s) in layer_s.items():
+          op(x_in[w.shape[1]], w, s, quantize_activation=qa)
+
+      _, ev, _ = time_calls([run_layer], 20, 5, use_graph)
+      extra[f"llama3_8b_layer_linears_{tag}"] = {"us": round(ev * 1e3, 2),
+                                                 "note": "weights (218 MB) stay cache-warm between iterations"}
+    result["extra"] = extra
+
+  # ---- CPU baseline: the oracle (reference's eager CPU semantics) on this host ----
+  if not args.no_cpu:
+    from oracle import quantized_matmul_oracle as oracle
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    oracle.quantized_matmul(x16, w_cpu, s_cpu)  # warm-up
+    t_runs = []
+    t_start = time.perf_counter()
+    while len(t_runs) < 5 or (time.perf_counter() - t_start < 10.0 and len(t_runs) < 50):
+      t0 = time.perf_counter()
+      oracle.quantized_matmul(x16, w_cpu, s_cpu)
+      t_runs.append(time.perf_counter() - t0)
+    t_med = sorted(t_runs)[len(t_runs) // 2]
+    result["cpu_baseline"] = {
+        "value": round(bytes16 / t_med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"median of {len(t_runs)} full calls of the same M=16 workload through the CPU oracle "
+                  f"(torch {torch.__version__} eager ops, the reference's CPU-tensor semantics); "
+                  f"{t_med * 1e3:.1f} ms per call",
+    }
+  print(json.dumps(result))
+
+
+if __name__ == "__main__":
+  main()

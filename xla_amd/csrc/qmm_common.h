@@ -21,6 +21,17 @@ static inline int qmm_dt_size(int dt) { return dt == XLA_AMD_DT_F32 ? 4 : 2; }
 __host__ __device__ static inline int qmm_promote(int a, int b) { return a == b ? a : XLA_AMD_DT_F32; }
 
 // ---- device side -----------------------------------------------------------
+// Compile-time loop: f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>).
+// Keeps register arrays indexed by constants where `#pragma unroll` gives up.
+template <int V> struct qmm_const { static constexpr int value = V; constexpr operator int() const { return V; } };
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void qmm_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(qmm_const<I>{});
+    qmm_static_for<N, I + 1>(f);
+  }
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));

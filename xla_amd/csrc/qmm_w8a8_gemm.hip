@@ -156,37 +156,39 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
 
   // Epilogue.
   const bool has_zp = g.zp != nullptr;
-#pragma unroll
-  for (int j = 0; j < NI; ++j) {
-    const int n = n0 + wn * TN + j * 32 + lrow;
-    const bool n_ok = n < g.N;
-    float ws = 0.f, zpv = 0.f;
-    if (g.out && n_ok) {
-      ws = qmm_load(g.w_scale, n, g.w_scale_dt);
-      if (has_zp) zpv = qmm_load(g.zp, n, g.zp_dt);
-    }
-#pragma unroll
-    for (int i = 0; i < MI; ++i) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * lchunk + (v & 3);
-        if (!n_ok || m >= g.M) continue;
-        const int a = acc[i][j][v];
-        const size_t idx = (size_t)m * g.N + n;
-        if (g.acc_out) g.acc_out[idx] = a;
-        if (g.out) {
-          float val = qmm_round_dt((float)a, g.cvt_dt);
-          val = qmm_round_dt(val * ws, g.mid_dt);
-          if (has_zp) {
-            float z = qmm_round_dt(qmm_round_dt((float)g.x_sum[m], g.zpo_dt) * zpv, g.zpo_dt);
-            val = qmm_round_dt(val - z, g.mid_dt);
-          }
-          val = qmm_round_dt(val * qmm_load(g.x_scale, m, g.x_scale_dt), g.out_dt);
-          qmm_store(g.out, idx, val, g.out_dt);
-        }
+  const bool want_out = g.out != nullptr, want_acc = g.acc_out != nullptr;
+  qmm_static_for<MI>([&](auto ic) {
+    constexpr int i = ic;
+    qmm_static_for<16>([&](auto vc) {
+      constexpr int v = vc;
+      const int m = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * lchunk + (v & 3);
+      const bool m_ok = m < g.M;
+      float xs = 0.f, xsum_f = 0.f;
+      if (want_out && m_ok) {
+        xs = qmm_load(g.x_scale, m, g.x_scale_dt);
+        if (has_zp) xsum_f = qmm_round_dt((float)g.x_sum[m], g.zpo_dt);
       }
-    }
-  }
+      qmm_static_for<NI>([&](auto jc) {
+        constexpr int j = jc;
+        const int n = n0 + wn * TN + j * 32 + lrow;
+        if (m_ok && n < g.N) {
+          const int a = acc[i][j][v];
+          const size_t idx = (size_t)m * g.N + n;
+          if (want_acc) g.acc_out[idx] = a;
+          if (want_out) {
+            float val = qmm_round_dt((float)a, g.cvt_dt);
+            val = qmm_round_dt(val * qmm_load(g.w_scale, n, g.w_scale_dt), g.mid_dt);
+            if (has_zp) {
+              float z = qmm_round_dt(xsum_f * qmm_load(g.zp, n, g.zp_dt), g.zpo_dt);
+              val = qmm_round_dt(val - z, g.mid_dt);
+            }
+            val = qmm_round_dt(val * xs, g.out_dt);
+            qmm_store(g.out, idx, val, g.out_dt);
+          }
+        }
+      });
+    });
+  });
 }
 
 template <int BM, int BN, int WM, int WN>
