@@ -148,46 +148,110 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   __syncthreads();
   for (int kt = 0; kt < ksteps; ++kt) {
     const int cur = kt & 1;
-    if (kt + 1 < ksteps) gload((kt + 1) * kBK);
-    compute(cur);
-    if (kt + 1 < ksteps) sstore(cur ^ 1);
-    __syncthreads();
+#ifndef QMM_DBG
+#define QMM_DBG 0
+#endif
+    if constexpr (!(QMM_DBG & 1)) { if (kt + 1 < ksteps) gload((kt + 1) * kBK); }
+    if constexpr (!(QMM_DBG & 2)) compute(cur);
+    if constexpr (!(QMM_DBG & 4)) { if (kt + 1 < ksteps) sstore(cur ^ 1); }
+    if constexpr (!(QMM_DBG & 8)) __syncthreads();
   }
 
-  // Epilogue.
+  // Epilogue, staged through LDS so that (a) the code stays small (the
+  // accumulators are register-indexed by constants only in the 16*MI*NI
+  // ds_write instructions; everything else is a rolled loop) and (b) global
+  // stores are row-contiguous vectors instead of one element per lane.
+  if constexpr (QMM_DBG & 16) { if (acc[0][0][0] != 12345) return; }
+  constexpr int kEpStride = TN + 8;  // ints per staged row: +8 keeps rows 16-byte aligned and
+                                     // shifts the second half-wave (4 rows down) by 32 banks
+  static_assert(4 * WM * WN * 32 * kEpStride + 4 * 4 * (BM + BN) <= 2 * (BM + BN) * kBK,
+                "epilogue staging must fit in the pipeline's LDS");
+  __syncthreads();  // every wave is done reading the last pipeline stage
+  float* s_xs = (float*)smem;          // [BM] activation scale
+  float* s_xsum = s_xs + BM;           // [BM] round_zpo(float(x_sum))
+  float* s_ws = s_xsum + BM;           // [BN] weight scale
+  float* s_zp = s_ws + BN;             // [BN] zero point
+  int* s_ep = (int*)(s_zp + BN) + wave * (32 * kEpStride);  // per-wave [32][kEpStride]
   const bool has_zp = g.zp != nullptr;
   const bool want_out = g.out != nullptr, want_acc = g.acc_out != nullptr;
+  if (want_out) {
+    for (int t = tid; t < BM; t += T) {
+      const int m = min(m0 + t, g.M - 1);
+      s_xs[t] = qmm_load(g.x_scale, m, g.x_scale_dt);
+      s_xsum[t] = has_zp ? qmm_round_dt((float)g.x_sum[m], g.zpo_dt) : 0.f;
+    }
+    for (int t = tid; t < BN; t += T) {
+      const int n = min(n0 + t, g.N - 1);
+      s_ws[t] = qmm_load(g.w_scale, n, g.w_scale_dt);
+      s_zp[t] = has_zp ? qmm_load(g.zp, n, g.zp_dt) : 0.f;
+    }
+  }
+  __syncthreads();
+  const bool simple = g.cvt_dt == XLA_AMD_DT_F32 && g.mid_dt == XLA_AMD_DT_F32 && !has_zp;
+  const bool n_vec = (g.N % 4) == 0;  // rows of out start 8/16-byte aligned
+  constexpr int kLanesPerRow = TN / 4;               // each lane finishes 4 consecutive n
+  constexpr int kPasses = 32 * kLanesPerRow / 64;    // passes over a 32-row block
+
+  // Finishes one staged 32 x TN block whose first row is global row mb.
+  auto finish_block = [&](int mb, int row_off) {
+    for (int p = 0; p < kPasses; ++p) {
+      const int idx = p * 64 + lane;
+      const int row = idx / kLanesPerRow, c4 = idx % kLanesPerRow;
+      const int m = mb + row, n = n0 + wn * TN + c4 * 4;
+      if (m >= g.M || n >= g.N) continue;
+      const i32x4 a = *(const i32x4*)(s_ep + row * kEpStride + c4 * 4);
+      const size_t idx0 = (size_t)m * g.N + n;
+      const int nvalid = min(4, g.N - n);
+      if (want_acc) {
+        if (n_vec) *(i32x4*)(g.acc_out + idx0) = a;
+        else for (int e = 0; e < nvalid; ++e) g.acc_out[idx0 + e] = a[e];
+      }
+      if (!want_out) continue;
+      const float xs = s_xs[row_off + row];
+      const f32x4 ws = *(const f32x4*)(s_ws + wn * TN + c4 * 4);
+      float val[4];
+      if (simple) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) val[e] = ((float)a[e] * ws[e]) * xs;
+      } else {
+        const float xsum_f = s_xsum[row_off + row];
+        const f32x4 zp4 = *(const f32x4*)(s_zp + wn * TN + c4 * 4);
+        for (int e = 0; e < 4; ++e) {
+          float v = qmm_round_dt((float)a[e], g.cvt_dt);
+          v = qmm_round_dt(v * ws[e], g.mid_dt);
+          if (has_zp) v = qmm_round_dt(v - qmm_round_dt(xsum_f * zp4[e], g.zpo_dt), g.mid_dt);
+          val[e] = v * xs;
+        }
+      }
+      if (g.out_dt == XLA_AMD_DT_F32) {
+        if (n_vec) *(f32x4*)((float*)g.out + idx0) = f32x4{val[0], val[1], val[2], val[3]};
+        else for (int e = 0; e < nvalid; ++e) ((float*)g.out)[idx0 + e] = val[e];
+      } else {
+        uint16_t h[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          h[e] = g.out_dt == XLA_AMD_DT_BF16 ? qmm_f32_to_bf16(val[e]) : qmm_f32_to_f16(val[e]);
+        if (n_vec) {
+          i32x2 pk = {(int)(h[0] | ((uint32_t)h[1] << 16)), (int)(h[2] | ((uint32_t)h[3] << 16))};
+          *(i32x2*)((uint16_t*)g.out + idx0) = pk;
+        } else {
+          for (int e = 0; e < nvalid; ++e) ((uint16_t*)g.out)[idx0 + e] = h[e];
+        }
+      }
+    }
+  };
+
   qmm_static_for<MI>([&](auto ic) {
     constexpr int i = ic;
-    qmm_static_for<16>([&](auto vc) {
-      constexpr int v = vc;
-      const int m = m0 + wm * TM + i * 32 + 8 * (v >> 2) + 4 * lchunk + (v & 3);
-      const bool m_ok = m < g.M;
-      float xs = 0.f, xsum_f = 0.f;
-      if (want_out && m_ok) {
-        xs = qmm_load(g.x_scale, m, g.x_scale_dt);
-        if (has_zp) xsum_f = qmm_round_dt((float)g.x_sum[m], g.zpo_dt);
-      }
-      qmm_static_for<NI>([&](auto jc) {
-        constexpr int j = jc;
-        const int n = n0 + wn * TN + j * 32 + lrow;
-        if (m_ok && n < g.N) {
-          const int a = acc[i][j][v];
-          const size_t idx = (size_t)m * g.N + n;
-          if (want_acc) g.acc_out[idx] = a;
-          if (want_out) {
-            float val = qmm_round_dt((float)a, g.cvt_dt);
-            val = qmm_round_dt(val * qmm_load(g.w_scale, n, g.w_scale_dt), g.mid_dt);
-            if (has_zp) {
-              float z = qmm_round_dt(xsum_f * qmm_load(g.zp, n, g.zp_dt), g.zpo_dt);
-              val = qmm_round_dt(val - z, g.mid_dt);
-            }
-            val = qmm_round_dt(val * xs, g.out_dt);
-            qmm_store(g.out, idx, val, g.out_dt);
-          }
-        }
+    qmm_static_for<NI>([&](auto jc) {
+      constexpr int j = jc;
+      qmm_static_for<16>([&](auto vc) {
+        constexpr int v = vc;
+        s_ep[(8 * (v >> 2) + 4 * lchunk + (v & 3)) * kEpStride + j * 32 + lrow] = acc[i][j][v];
       });
     });
+    // LDS operations of one wave complete in order: the reads below see the writes above.
+    finish_block(m0 + wm * TM + i * 32, wm * TM + i * 32);
   });
 }
 
