@@ -21,11 +21,6 @@ constexpr int kWaves = 4;    // waves per workgroup (K is split over them)
 constexpr int kKIter = 128;  // k columns per wave iteration
 
 // ---- operand fragments --------------------------------------------------------
-// Fragment of 8 k-values for one MFMA, per x dtype.
-template <int XT> struct Frag;
-template <> struct Frag<XLA_AMD_DT_BF16> { typedef bf16x8 T; };
-template <> struct Frag<XLA_AMD_DT_F16> { typedef f16x8 T; };
-
 __device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
   // {bf16(lo), bf16(hi)} by truncation: exact for integers of magnitude <= 256.
   return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
@@ -106,18 +101,21 @@ struct SkinnyArgs {
 };
 
 // XT: dtype of x.  BITS: 8 or 4.  MT: 16-row tiles of x.  RG: 16-channel
-// groups per wave.  PERCH: per-channel (C == K): waves interleave over k and
-// raw dot products are reduced; otherwise each wave owns whole blocks and the
-// reduction is over scaled block results.  NEEDXS: x sums are needed (zero
-// point and/or the int4 affine map).
-template <int XT, int BITS, int MT, int RG, bool PERCH, bool HASZP>
+// groups per wave.  D: k-iterations whose loads are in flight per wave (a
+// register ring: iteration j lives in stage j % D).  PERCH: per-channel
+// (C == K): waves interleave over k and raw dot products are reduced;
+// otherwise each wave owns whole blocks and the reduction is over scaled block
+// results.  HASZP: a zero point is given.
+template <int XT, int BITS, int MT, int RG, int D, bool PERCH, bool HASZP>
 __global__ void __launch_bounds__(kWaves * 64)
 qmm_skinny_kernel(SkinnyArgs a) {
   constexpr bool kMfma = XT != XLA_AMD_DT_F32;
-  constexpr bool NEEDXS = HASZP || (BITS == 4 && kMfma);
+  constexpr bool NEEDXS = HASZP || (BITS == 4 && kMfma);  // x sums: zero point, int4 affine map
   constexpr int kSlots = RG * MT * 4;                 // accumulators per lane
   constexpr int kXsSlots = NEEDXS ? MT : 0;           // x sums per lane (PERCH reduce)
   constexpr int kRedSlots = PERCH ? kSlots + kXsSlots : (HASZP ? 2 * kSlots : kSlots);
+  constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte weight loads per lane per iteration
+  constexpr int XQ = kMfma ? 4 : 8;                   // 16-byte x loads per lane per iteration
   __shared__ float red[kWaves][kRedSlots][64];
 
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -142,7 +140,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   }
 
   f32x4 acc[RG][MT];
-  f32x4 xs[MT > 0 ? MT : 1];
+  f32x4 xs[MT];
   f32x4 sacc[RG][MT], zacc[RG][MT];
 #pragma unroll
   for (int rg = 0; rg < RG; ++rg)
@@ -155,76 +153,93 @@ qmm_skinny_kernel(SkinnyArgs a) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xs[mt] = f32x4{0, 0, 0, 0};
 
-  // One k-iteration: 128 columns starting at k0.
-  auto iterate = [&](int k0) {
-    // Issue all loads first.
-    i32x4 wq[RG][BITS == 8 ? 2 : 1];
+  // Iteration j of this wave -> first column k0.  Per-channel: iterations are
+  // dealt round-robin to the waves.  Blockwise: blocks are dealt round-robin
+  // and a wave walks its block's C/128 iterations consecutively.
+  const int ipb = PERCH ? 1 : a.C / kKIter;  // iterations per block
+  const int units = PERCH ? K / kKIter : K / a.C;     // iterations resp. blocks in total
+  const int my_units = units > wv ? (units - wv + kWaves - 1) / kWaves : 0;
+  const int n_it = my_units * ipb;
+  // Workgroups start at different k (rotation `rot`): rows are K bytes apart,
+  // so without it every wave of the grid would begin in the same few hundred
+  // bytes of each row and crowd the same memory channels.
+  const int rot = (int)((blockIdx.x * 5u) % (unsigned)units);
+  auto unit_of = [&](int u) -> int {  // u-th unit of this wave -> global unit index
+    int t = wv + u * kWaves + rot;
+    return t >= units ? t - units : t;
+  };
+  auto k0_of = [&](int j) -> int {
+    if constexpr (PERCH) return unit_of(j) * kKIter;
+    const int b = j / ipb, i = j - b * ipb;
+    return unit_of(b) * a.C + i * kKIter;
+  };
+
+  // Register ring of D stages.
+  i32x4 wq[D][RG][WQ];
+  i32x4 xq[D][MT][XQ];
+  auto load_stage = [&](auto dc, int j) {
+    constexpr int d = dc;
+    const int k0 = k0_of(j);
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
-      if constexpr (BITS == 8) {
-        const i32x4* p = (const i32x4*)(wrow[rg] + k0);
-        wq[rg][0] = __builtin_nontemporal_load(p);
-        wq[rg][1] = __builtin_nontemporal_load(p + 1);
-      } else {
-        wq[rg][0] = __builtin_nontemporal_load((const i32x4*)(wrow[rg] + k0 / 2));
-      }
+      const i32x4* p = (const i32x4*)(wrow[rg] + (BITS == 8 ? k0 : k0 / 2));
+#pragma unroll
+      for (int q = 0; q < WQ; ++q) wq[d][rg][q] = __builtin_nontemporal_load(p + q);
     }
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const i32x4* p = (const i32x4*)(xrow[mt] + (size_t)k0 * (XT == XLA_AMD_DT_F32 ? 4 : 2));
+#pragma unroll
+      for (int q = 0; q < XQ; ++q) xq[d][mt][q] = p[q];
+    }
+  };
+
+  auto compute_stage = [&](auto dc) {
+    constexpr int d = dc;
     if constexpr (kMfma) {
-      i32x4 xf[MT][4];
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const i32x4* p = (const i32x4*)(xrow[mt] + (size_t)k0 * 2);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xf[mt][j] = p[j];
-      }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg) {
           i32x4 af;
           if constexpr (BITS == 8)
-            af = cvt_w8<XT>((uint32_t)wq[rg][j >> 1][(j & 1) * 2], (uint32_t)wq[rg][j >> 1][(j & 1) * 2 + 1]);
+            af = cvt_w8<XT>((uint32_t)wq[d][rg][j >> 1][(j & 1) * 2], (uint32_t)wq[d][rg][j >> 1][(j & 1) * 2 + 1]);
           else
-            af = cvt_w4<XT>((uint32_t)wq[rg][0][j]);
+            af = cvt_w4<XT>((uint32_t)wq[d][rg][0][j]);
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) acc[rg][mt] = mfma16<XT>(af, xf[mt][j], acc[rg][mt]);
+          for (int mt = 0; mt < MT; ++mt) acc[rg][mt] = mfma16<XT>(af, xq[d][mt][j], acc[rg][mt]);
         }
         if constexpr (NEEDXS) {
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) xs[mt] = mfma16<XT>(ones_frag<XT>(), xf[mt][j], xs[mt]);
+          for (int mt = 0; mt < MT; ++mt) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[d][mt][j], xs[mt]);
         }
       }
     } else {
       // f32 x: 16x16x4 f32 MFMA, one k per lane per instruction.
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        f32x4 xv[MT];
+      for (int kk = 0; kk < 32; ++kk) {  // 0..31 within the lane's columns
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xv[mt] = ((const f32x4*)(xrow[mt] + (size_t)k0 * 4))[q];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          int kk = 4 * q + e;  // 0..31 within the lane's columns
-#pragma unroll
-          for (int rg = 0; rg < RG; ++rg) {
-            float wf;
-            if constexpr (BITS == 8) {
-              uint32_t d = (uint32_t)wq[rg][kk >> 4][(kk >> 2) & 3];
-              wf = (float)(int8_t)(d >> (8 * (kk & 3)));
-            } else {
-              // column kk = 8*word + P[nibble]: nibble = (c&1)*4 + (c>>1), c = kk % 8
-              uint32_t d = (uint32_t)wq[rg][0][kk >> 3];
-              int c = kk & 7, nib = (c & 1) * 4 + (c >> 1);
-              wf = (float)(int)((d >> (4 * nib)) & 15u) - 8.0f;
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-              acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv[mt][e], acc[rg][mt], 0, 0, 0);
+        for (int rg = 0; rg < RG; ++rg) {
+          float wf;
+          if constexpr (BITS == 8) {
+            uint32_t dw = (uint32_t)wq[d][rg][kk >> 4][(kk >> 2) & 3];
+            wf = (float)(int8_t)(dw >> (8 * (kk & 3)));
+          } else {
+            // column kk = 8*word + P[nibble]: nibble = (c&1)*4 + (c>>1), c = kk % 8
+            uint32_t dw = (uint32_t)wq[d][rg][0][kk >> 3];
+            int c = kk & 7, nib = (c & 1) * 4 + (c >> 1);
+            wf = (float)(int)((dw >> (4 * nib)) & 15u) - 8.0f;
           }
-          if constexpr (NEEDXS) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-              xs[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, xv[mt][e], xs[mt], 0, 0, 0);
-          }
+          for (int mt = 0; mt < MT; ++mt)
+            acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                wf, __builtin_bit_cast(float, xq[d][mt][kk >> 2][kk & 3]), acc[rg][mt], 0, 0, 0);
+        }
+        if constexpr (NEEDXS) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            xs[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(
+                1.0f, __builtin_bit_cast(float, xq[d][mt][kk >> 2][kk & 3]), xs[mt], 0, 0, 0);
         }
       }
     }
@@ -236,10 +251,51 @@ qmm_skinny_kernel(SkinnyArgs a) {
     return accv;
   };
 
+  // Block epilogue (blockwise only): p = round_x(dot); sacc += scale[s,n] * p;
+  // zacc += round_x(xsum) * zp[s,n]; then the block accumulators restart.
+  auto block_epilogue = [&](int sblk) {
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        int n = min(n_base + 16 * rg + 4 * g + v, N - 1);
+        float sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
+        float zv = 0.f;
+        if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          float xsv = NEEDXS ? xs[mt][v] : 0.f;
+          float p = qmm_round_dt(true_dot(acc[rg][mt][v], xsv), x_dt);
+          sacc[rg][mt][v] = fmaf(sc, p, sacc[rg][mt][v]);
+          if constexpr (HASZP) zacc[rg][mt][v] = fmaf(qmm_round_dt(xsv, x_dt), zv, zacc[rg][mt][v]);
+        }
+      }
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[rg][mt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) xs[mt] = f32x4{0, 0, 0, 0};
+  };
+
+  // Software pipeline: D iterations of loads stay in flight.
+  qmm_static_for<D>([&](auto dc) {
+    if (dc < n_it) load_stage(dc, dc);
+  });
+  for (int j0 = 0; j0 < n_it; j0 += D) {
+    qmm_static_for<D>([&](auto dc) {
+      const int j = j0 + dc;
+      if (j < n_it) {
+        compute_stage(dc);
+        if (j + D < n_it) load_stage(dc, j + D);
+        if constexpr (!PERCH) {
+          if ((j + 1) % ipb == 0) block_epilogue(unit_of(j / ipb));
+        }
+      }
+    });
+  }
+
   if constexpr (PERCH) {
-    const int iters = K / kKIter;
-#pragma unroll 2
-    for (int it = wv; it < iters; it += kWaves) iterate(it * kKIter);
     // Reduce raw partial sums over the waves.
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg)
@@ -252,33 +308,6 @@ qmm_skinny_kernel(SkinnyArgs a) {
       for (int mt = 0; mt < MT; ++mt) red[wv][kSlots + mt][lane] = xs[mt][0];
     }
   } else {
-    const int S = K / a.C, ipb = a.C / kKIter;
-    for (int s = wv; s < S; s += kWaves) {
-      for (int i = 0; i < ipb; ++i) iterate(s * a.C + i * kKIter);
-      // Block epilogue: p = round_x(dot); sacc += scale[s,n] * p; zacc += round_x(xsum) * zp[s,n].
-#pragma unroll
-      for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          int n = min(n_base + 16 * rg + 4 * g + v, N - 1);
-          float sc = qmm_load(a.scale, (int64_t)s * N + n, a.scale_dt);
-          float zv = 0.f;
-          if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)s * N + n, a.zp_dt);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            float xsv = NEEDXS ? xs[mt][v] : 0.f;
-            float p = qmm_round_dt(true_dot(acc[rg][mt][v], xsv), x_dt);
-            sacc[rg][mt][v] = fmaf(sc, p, sacc[rg][mt][v]);
-            if constexpr (HASZP) zacc[rg][mt][v] = fmaf(qmm_round_dt(xsv, x_dt), zv, zacc[rg][mt][v]);
-          }
-        }
-#pragma unroll
-      for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) acc[rg][mt] = f32x4{0, 0, 0, 0};
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xs[mt] = f32x4{0, 0, 0, 0};
-    }
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
@@ -326,11 +355,26 @@ qmm_skinny_kernel(SkinnyArgs a) {
   }
 }
 
+#ifndef QMM_SKINNY_RG
+#define QMM_SKINNY_RG 1
+#endif
+#ifndef QMM_SKINNY_D
+#define QMM_SKINNY_D 0
+#endif
+
+// Pipeline depth: as many iterations in flight as ~150 VGPRs of staging allow.
+constexpr int pipeline_depth(int xt, int mt) {
+  if (QMM_SKINNY_D > 0) return QMM_SKINNY_D;
+  if (xt == XLA_AMD_DT_F32) return mt <= 2 ? 2 : 1;
+  return mt == 1 ? 4 : (mt == 2 ? 3 : 2);
+}
+
 template <int XT, int BITS, int MT, bool PERCH, bool HASZP>
 int launch_rg(const SkinnyArgs& a, hipStream_t stream) {
-  constexpr int RG = 1;
+  constexpr int RG = QMM_SKINNY_RG;
+  constexpr int D = pipeline_depth(XT, MT);
   unsigned blocks = (unsigned)((a.N + 16 * RG - 1) / (16 * RG));
-  hipLaunchKernelGGL((qmm_skinny_kernel<XT, BITS, MT, RG, PERCH, HASZP>), dim3(blocks),
+  hipLaunchKernelGGL((qmm_skinny_kernel<XT, BITS, MT, RG, D, PERCH, HASZP>), dim3(blocks),
                      dim3(kWaves * 64), 0, stream, a);
   return QMM_CHECK_LAUNCH("weight_only_skinny launch");
 }
