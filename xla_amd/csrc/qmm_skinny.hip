@@ -1,24 +1,35 @@
 // Weight-streaming GEMV / skinny GEMM for weight-only quantized linear layers
-// on gfx950.  HBM-bound: every weight byte is read once with 128-bit loads,
-// converted in registers and fed to MFMA against up to 64 rows of x that stay
-// in registers; K is split over the waves of a workgroup and reduced in LDS.
+// on gfx950.  HBM-bound: every weight byte is read from memory exactly once.
 //
-// Thread/data mapping.  A workgroup owns 16*RG consecutive output channels
-// (rows n of the K-major weight).  Lane l of a wave is (r = l%16, g = l/16):
-// in one k-iteration of 128 columns it loads, for row n0+r, the 32 weights at
-// columns k0+32g..k0+32g+31 (32 bytes for int8, 16 bytes for int4), and for x
-// row m = r of each 16-row tile the same 32 columns.  The 32 columns go
-// through four 16x16x32 MFMAs (A = weights: 16 channels x 32 k, B = x^T:
-// 32 k x 16 rows), each lane contributing 8 k per MFMA for both operands, so
-// any k-order the hardware uses inside the instruction pairs the same
-// elements.  D[i][j] lands in lane (j + 16*(i/4)), register i%4:
-// channel n0 + 4g + v, x row r.
+// Memory access.  Global loads are issued so that one wave instruction reads
+// long contiguous runs (2 weight rows x 512 B, or 1 KB of one x row): that is
+// what the memory system streams fastest.  The matrix cores want the opposite
+// arrangement (lane = row, 8 consecutive k per lane), so tiles take one trip
+// through LDS: written as they were loaded, read back in MFMA operand order.
+// 16-byte chunks are XOR-swizzled with the row number so that both directions
+// are free of bank conflicts.
+//
+// Work split.  A workgroup has 4 waves arranged as RW row groups x KW k-splits
+// (RW * KW == 4).  It owns 16*RW consecutive output channels.  K is walked in
+// steps of KS columns per k-split (512 B of weight row: 512 columns of int8,
+// 1024 of int4); wave (rw, kw) handles steps kw, kw + KW, ...  The x tile of a
+// step ([16*MT rows] x KS columns) is shared by the RW waves of a k-split.
+// Large N uses RW = 4 (no cross-wave reduction at all); small N trades row
+// groups for k-splits so that the grid still covers the chip.
+//
+// MFMA mapping.  Lane l is (r = l%16, g = l/16).  For a sub-step of 128
+// columns the lane supplies, for weight row r and for x row r of each 16-row
+// tile, the 32 columns k0+32g..k0+32g+31, as four 16x16x32 MFMAs of 8 columns
+// per lane (A = weights, B = x^T).  Both operands use the same columns per
+// lane, so the k-order inside the instruction does not matter.  D[i][j] lands
+// in lane (j + 16*(i/4)), register i%4: channel 4g + v, x row r.
 #include "qmm_common.h"
 
 namespace {
 
-constexpr int kWaves = 4;    // waves per workgroup (K is split over them)
-constexpr int kKIter = 128;  // k columns per wave iteration
+constexpr int kWaves = 4;
+constexpr int kWSeg = 512;        // weight bytes per row per step
+constexpr int kLdsLimit = 160 * 1024;
 
 // ---- operand fragments --------------------------------------------------------
 __device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
@@ -52,7 +63,7 @@ __device__ __forceinline__ i32x4 cvt_w8(uint32_t d0, uint32_t d1) {
   return o;
 }
 
-// 8 packed int4 weights (one dword, nibble j = column P[j] + 8 biased) -> 8
+// 8 packed int4 weights (one dword, nibble j = column P[j], biased by 8) -> 8
 // elements (1 + u/16) of the x dtype, u = w + 8 in 0..15.  The caller undoes
 // the affine map with the exact x sum: sum w*x = 16*(sum a*x - 1.5*sum x).
 template <int XT>
@@ -100,301 +111,431 @@ struct SkinnyArgs {
   int scale_dt, zp_dt, out_dt;
 };
 
-// XT: dtype of x.  BITS: 8 or 4.  MT: 16-row tiles of x.  RG: 16-channel
-// groups per wave.  D: k-iterations whose loads are in flight per wave (a
-// register ring: iteration j lives in stage j % D).  PERCH: per-channel
-// (C == K): waves interleave over k and raw dot products are reduced;
-// otherwise each wave owns whole blocks and the reduction is over scaled block
-// results.  HASZP: a zero point is given.
-template <int XT, int BITS, int MT, int RG, int D, bool PERCH, bool HASZP>
+// Reduction over the k-splits of a workgroup.
+constexpr int kRedNone = 0;    // blockwise, KW == 1: nothing to reduce
+constexpr int kRedRaw = 1;     // per-channel (C == K, any KW): raw dot products and x sums are summed, then scaled
+constexpr int kRedScaled = 2;  // blockwise, KW > 1, whole blocks per step (KS % C == 0): scaled block results are summed
+
+template <int XT, int BITS, int MT, int KW>
+struct SkinnyCfg {
+  static constexpr int RW = kWaves / KW;
+  static constexpr int XB = XT == XLA_AMD_DT_F32 ? 4 : 2;
+  static constexpr int KS = BITS == 8 ? kWSeg : 2 * kWSeg;  // columns per step
+  static constexpr int SUB = KS / 128;                       // 128-column sub-steps per step
+  static constexpr int XROW = KS * XB;                       // bytes of one x row per step
+  static constexpr int XROWS = 16 * MT;
+  static constexpr int W_TILE = kWaves * 16 * kWSeg;         // 32 KB: every wave's 16 rows x 512 B
+  static constexpr int X_TILE = XROWS * XROW;                // per k-split
+  static constexpr int STAGE = W_TILE + KW * X_TILE;
+  static constexpr int NS = 2 * STAGE <= kLdsLimit ? 2 : 1;  // LDS stages
+  static constexpr int XP = X_TILE / 1024 / RW;              // 1 KB x loads per wave per step
+  static constexpr int P = (32 + 4 * XP) <= 64 ? 2 : 1;      // steps of loads in flight (register ring)
+  static constexpr int LDS_BYTES = NS * STAGE;
+  static constexpr bool kFits = STAGE <= kLdsLimit;
+  static_assert((X_TILE / 1024) % RW == 0, "x tile must split evenly over the waves of a k-split");
+};
+
+template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
 __global__ void __launch_bounds__(kWaves * 64)
 qmm_skinny_kernel(SkinnyArgs a) {
+  using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
+  constexpr int RW = Cfg::RW, XB = Cfg::XB, KS = Cfg::KS, SUB = Cfg::SUB, XROW = Cfg::XROW;
+  constexpr int W_TILE = Cfg::W_TILE, X_TILE = Cfg::X_TILE, STAGE = Cfg::STAGE, NS = Cfg::NS;
+  constexpr int XP = Cfg::XP, P = Cfg::P;
   constexpr bool kMfma = XT != XLA_AMD_DT_F32;
   constexpr bool NEEDXS = HASZP || (BITS == 4 && kMfma);  // x sums: zero point, int4 affine map
-  constexpr int kSlots = RG * MT * 4;                 // accumulators per lane
-  constexpr int kXsSlots = NEEDXS ? MT : 0;           // x sums per lane (PERCH reduce)
-  constexpr int kRedSlots = PERCH ? kSlots + kXsSlots : (HASZP ? 2 * kSlots : kSlots);
-  constexpr int WQ = BITS == 8 ? 2 : 1;               // 16-byte weight loads per lane per iteration
-  constexpr int XQ = kMfma ? 4 : 8;                   // 16-byte x loads per lane per iteration
-  __shared__ float red[kWaves][kRedSlots][64];
+  constexpr int XQ = kMfma ? 4 : 8;                       // 16-byte x chunks per lane per sub-step
+  extern __shared__ __attribute__((aligned(16))) char smem[];
 
-  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rw = wave % RW, kw = wave / RW;
   const int r = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.x * (16 * RG);
-  const int K = a.K, N = a.N, M = a.M;
+  const int K = a.K, N = a.N, M = a.M, C = a.C;
+  const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
+  const int row_bytes = BITS == 8 ? K : K / 2;          // bytes of one weight row
   const int x_dt = XT;
 
-  // Row pointers (clamped so that tail lanes read valid memory; their results
-  // are never stored).
-  const uint8_t* wrow[RG];
-#pragma unroll
-  for (int rg = 0; rg < RG; ++rg) {
-    int n = min(n_base + 16 * rg + r, N - 1);
-    wrow[rg] = a.w + (size_t)n * (BITS == 8 ? (size_t)K : (size_t)K / 2) + (BITS == 8 ? 32 * g : 16 * g);
-  }
-  const char* xrow[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int m = min(16 * mt + r, M - 1);
-    xrow[mt] = (const char*)a.x + ((size_t)m * K + 32 * g) * (XT == XLA_AMD_DT_F32 ? 4 : 2);
-  }
+  // ---- global -> register loads (coalesced) ------------------------------------
+  // Addresses are a workgroup-uniform base (scalar registers, advanced per step
+  // with scalar arithmetic) plus a per-lane 32-bit offset that never changes.
+  // weights: instruction i covers rows 2i, 2i+1 of the wave's 16, 512 B each
+  const int n_wg = blockIdx.x * (16 * RW);
+  const uint8_t* const w_base = a.w + (size_t)n_wg * row_bytes;
+  const char* const x_base = (const char*)a.x;
+  const int w_lrow = lane >> 5, w_chunk = lane & 31;
+  uint32_t w_off[8];
+  int w_dst[8];
+  qmm_static_for<8>([&](auto ic) {
+    constexpr int i = ic;
+    const int row = 2 * i + w_lrow;
+    const int n = min(n_wave + row, N - 1);  // tail rows read the last valid row
+    w_off[i] = (uint32_t)(n - n_wg) * (uint32_t)row_bytes + w_chunk * 16;
+    w_dst[i] = wave * (16 * kWSeg) + row * kWSeg + ((w_chunk ^ row) * 16);
+  });
+  // x: piece j of this wave is 1 KB of one row of the k-split's tile
+  uint32_t x_off[XP];
+  int x_dst[XP];
+  qmm_static_for<XP>([&](auto jc) {
+    constexpr int j = jc;
+    constexpr int kPiecesPerRow = XROW / 1024;
+    const int q = rw * XP + j;
+    const int row = q / kPiecesPerRow, chunk = (q % kPiecesPerRow) * 64 + lane;
+    const int m = min(row, M - 1);
+    x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + chunk * 16;
+    x_dst[j] = W_TILE + kw * X_TILE + row * XROW + ((chunk ^ (row & 15)) * 16);
+  });
 
-  f32x4 acc[RG][MT];
-  f32x4 xs[MT];
-  f32x4 sacc[RG][MT], zacc[RG][MT];
-#pragma unroll
-  for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      acc[rg][mt] = f32x4{0, 0, 0, 0};
-      sacc[rg][mt] = f32x4{0, 0, 0, 0};
-      zacc[rg][mt] = f32x4{0, 0, 0, 0};
-    }
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xs[mt] = f32x4{0, 0, 0, 0};
+  const int steps_total = (K + KS - 1) / KS;
+  const int my_steps = steps_total > kw ? (steps_total - kw + KW - 1) / KW : 0;
+  // every wave of the workgroup runs the same number of loop trips (barriers)
+  const int trips = (steps_total + KW - 1) / KW;
 
-  // Iteration j of this wave -> first column k0.  Per-channel: iterations are
-  // dealt round-robin to the waves.  Blockwise: blocks are dealt round-robin
-  // and a wave walks its block's C/128 iterations consecutively.
-  const int ipb = PERCH ? 1 : a.C / kKIter;  // iterations per block
-  const int units = PERCH ? K / kKIter : K / a.C;     // iterations resp. blocks in total
-  const int my_units = units > wv ? (units - wv + kWaves - 1) / kWaves : 0;
-  const int n_it = my_units * ipb;
-  // Workgroups start at different k (rotation `rot`): rows are K bytes apart,
-  // so without it every wave of the grid would begin in the same few hundred
-  // bytes of each row and crowd the same memory channels.
-  const int rot = (int)((blockIdx.x * 5u) % (unsigned)units);
-  auto unit_of = [&](int u) -> int {  // u-th unit of this wave -> global unit index
-    int t = wv + u * kWaves + rot;
-    return t >= units ? t - units : t;
-  };
-  auto k0_of = [&](int j) -> int {
-    if constexpr (PERCH) return unit_of(j) * kKIter;
-    const int b = j / ipb, i = j - b * ipb;
-    return unit_of(b) * a.C + i * kKIter;
-  };
-
-  // Register ring of D stages.
-  i32x4 wq[D][RG][WQ];
-  i32x4 xq[D][MT][XQ];
-  auto load_stage = [&](auto dc, int j) {
-    constexpr int d = dc;
-    const int k0 = k0_of(j);
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg) {
-      const i32x4* p = (const i32x4*)(wrow[rg] + (BITS == 8 ? k0 : k0 / 2));
-#pragma unroll
-      for (int q = 0; q < WQ; ++q) wq[d][rg][q] = __builtin_nontemporal_load(p + q);
-    }
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const i32x4* p = (const i32x4*)(xrow[mt] + (size_t)k0 * (XT == XLA_AMD_DT_F32 ? 4 : 2));
-#pragma unroll
-      for (int q = 0; q < XQ; ++q) xq[d][mt][q] = p[q];
-    }
-  };
-
-  auto compute_stage = [&](auto dc) {
-    constexpr int d = dc;
-    if constexpr (kMfma) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int rg = 0; rg < RG; ++rg) {
-          i32x4 af;
-          if constexpr (BITS == 8)
-            af = cvt_w8<XT>((uint32_t)wq[d][rg][j >> 1][(j & 1) * 2], (uint32_t)wq[d][rg][j >> 1][(j & 1) * 2 + 1]);
-          else
-            af = cvt_w4<XT>((uint32_t)wq[d][rg][0][j]);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) acc[rg][mt] = mfma16<XT>(af, xq[d][mt][j], acc[rg][mt]);
-        }
-        if constexpr (NEEDXS) {
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[d][mt][j], xs[mt]);
-        }
-      }
+  i32x4 wreg[P][8];
+  i32x4 xreg[P][XP];
+  auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {  // s: this wave's s-th step
+    constexpr int p = pc;
+    const int gs = s * KW + kw;  // global step
+    const uint8_t* const wp = w_base + (size_t)gs * kWSeg;
+    const char* const xp = x_base + (size_t)gs * XROW;
+    if ((gs + 1) * KS <= K) {  // whole step inside K: no per-lane conditions
+      qmm_static_for<8>([&](auto ic) {
+        constexpr int i = ic;
+        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
+      });
+      qmm_static_for<XP>([&](auto jc) {
+        constexpr int j = jc;
+        xreg[p][j] = *(const i32x4*)(xp + x_off[j]);
+      });
     } else {
-      // f32 x: 16x16x4 f32 MFMA, one k per lane per instruction.
-#pragma unroll
-      for (int kk = 0; kk < 32; ++kk) {  // 0..31 within the lane's columns
-#pragma unroll
-        for (int rg = 0; rg < RG; ++rg) {
-          float wf;
-          if constexpr (BITS == 8) {
-            uint32_t dw = (uint32_t)wq[d][rg][kk >> 4][(kk >> 2) & 3];
-            wf = (float)(int8_t)(dw >> (8 * (kk & 3)));
-          } else {
-            // column kk = 8*word + P[nibble]: nibble = (c&1)*4 + (c>>1), c = kk % 8
-            uint32_t dw = (uint32_t)wq[d][rg][0][kk >> 3];
-            int c = kk & 7, nib = (c & 1) * 4 + (c >> 1);
-            wf = (float)(int)((dw >> (4 * nib)) & 15u) - 8.0f;
-          }
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            acc[rg][mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                wf, __builtin_bit_cast(float, xq[d][mt][kk >> 2][kk & 3]), acc[rg][mt], 0, 0, 0);
-        }
-        if constexpr (NEEDXS) {
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt)
-            xs[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(
-                1.0f, __builtin_bit_cast(float, xq[d][mt][kk >> 2][kk & 3]), xs[mt], 0, 0, 0);
-        }
-      }
+      // last, partial step: columns past K re-read the last valid 16 bytes of the
+      // row (their sub-steps are never computed)
+      const int w_left = row_bytes - gs * kWSeg, x_left = K * XB - gs * XROW;
+      qmm_static_for<8>([&](auto ic) {
+        constexpr int i = ic;
+        const uint32_t back = (uint32_t)max(w_chunk * 16 + 16 - w_left, 0);
+        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + (w_off[i] - back)));
+      });
+      qmm_static_for<XP>([&](auto jc) {
+        constexpr int j = jc;
+        constexpr int kPiecesPerRow = XROW / 1024;
+        const int col = (((rw * XP + j) % kPiecesPerRow) * 64 + lane) * 16;
+        const uint32_t back = (uint32_t)max(col + 16 - x_left, 0);
+        xreg[p][j] = *(const i32x4*)(xp + (x_off[j] - back));
+      });
     }
   };
+  auto store_lds = [&](auto pc, int stage) __attribute__((always_inline)) {
+    constexpr int p = pc;
+    char* base = smem + stage * STAGE;
+    qmm_static_for<8>([&](auto ic) {
+      constexpr int i = ic;
+      *(i32x4*)(base + w_dst[i]) = wreg[p][i];
+    });
+    qmm_static_for<XP>([&](auto jc) {
+      constexpr int j = jc;
+      *(i32x4*)(base + x_dst[j]) = xreg[p][j];
+    });
+  };
+
+  // ---- accumulators ----------------------------------------------------------------
+  // (register arrays are only ever indexed by compile-time constants: every
+  // loop over them is a qmm_static_for)
+  // acc/accb: two interleaved accumulation chains per tile (dependent MFMAs
+  // would otherwise wait for each other); their sum is the dot product.
+  f32x4 acc[MT], accb[MT], xs[MT], sacc[MT], zacc[MT];
+  qmm_static_for<MT>([&](auto mc) {
+    constexpr int mt = mc;
+    acc[mt] = f32x4{0, 0, 0, 0};
+    accb[mt] = f32x4{0, 0, 0, 0};
+    xs[mt] = f32x4{0, 0, 0, 0};
+    sacc[mt] = f32x4{0, 0, 0, 0};
+    zacc[mt] = f32x4{0, 0, 0, 0};
+  });
 
   // Undo the int4 affine map (MFMA path only): dot = 16 * (acc - 1.5 * xsum).
-  auto true_dot = [&](float accv, float xsv) -> float {
+  auto true_dot = [&](float accv, float xsv) __attribute__((always_inline)) -> float {
     if constexpr (BITS == 4 && kMfma) return 16.0f * (accv - 1.5f * xsv);
     return accv;
   };
 
-  // Block epilogue (blockwise only): p = round_x(dot); sacc += scale[s,n] * p;
-  // zacc += round_x(xsum) * zp[s,n]; then the block accumulators restart.
-  auto block_epilogue = [&](int sblk) {
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        int n = min(n_base + 16 * rg + 4 * g + v, N - 1);
-        float sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
-        float zv = 0.f;
-        if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          float xsv = NEEDXS ? xs[mt][v] : 0.f;
-          float p = qmm_round_dt(true_dot(acc[rg][mt][v], xsv), x_dt);
-          sacc[rg][mt][v] = fmaf(sc, p, sacc[rg][mt][v]);
-          if constexpr (HASZP) zacc[rg][mt][v] = fmaf(qmm_round_dt(xsv, x_dt), zv, zacc[rg][mt][v]);
-        }
-      }
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) acc[rg][mt] = f32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xs[mt] = f32x4{0, 0, 0, 0};
+  // End of quantization block sblk: p = round_x(dot); sacc += scale[s,n] * p;
+  // zacc += round_x(xsum) * zp[s,n]; the block accumulators restart.
+  auto block_epilogue = [&](int sblk) __attribute__((always_inline)) {
+    qmm_static_for<4>([&](auto vc) {
+      constexpr int v = vc;
+      const int n = min(n_wave + 4 * g + v, N - 1);
+      const float sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
+      float zv = 0.f;
+      if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
+      qmm_static_for<MT>([&](auto mc) {
+        constexpr int mt = mc;
+        const float xsv = NEEDXS ? xs[mt][v] : 0.f;
+        const float p = qmm_round_dt(true_dot(acc[mt][v] + accb[mt][v], xsv), x_dt);
+        sacc[mt][v] = fmaf(sc, p, sacc[mt][v]);
+        if constexpr (HASZP) zacc[mt][v] = fmaf(qmm_round_dt(xsv, x_dt), zv, zacc[mt][v]);
+      });
+    });
+    qmm_static_for<MT>([&](auto mc) {
+      constexpr int mt = mc;
+      acc[mt] = f32x4{0, 0, 0, 0};
+      accb[mt] = f32x4{0, 0, 0, 0};
+      xs[mt] = f32x4{0, 0, 0, 0};
+    });
   };
 
-  // Software pipeline: D iterations of loads stay in flight.
-  qmm_static_for<D>([&](auto dc) {
-    if (dc < n_it) load_stage(dc, dc);
-  });
-  for (int j0 = 0; j0 < n_it; j0 += D) {
-    qmm_static_for<D>([&](auto dc) {
-      const int j = j0 + dc;
-      if (j < n_it) {
-        compute_stage(dc);
-        if (j + D < n_it) load_stage(dc, j + D);
-        if constexpr (!PERCH) {
-          if ((j + 1) % ipb == 0) block_epilogue(unit_of(j / ipb));
+  // ---- one step out of LDS -----------------------------------------------------------
+  // Sub-steps (128 columns) left in the current quantization block; uniform.
+  const int sub_per_block = C / 128;
+  int block_left = sub_per_block;
+  auto compute = [&](auto fullc, int stage, int s) __attribute__((always_inline)) {
+    constexpr bool kFull = fullc != 0;  // the whole step lies inside K
+    const char* wb = smem + stage * STAGE + wave * (16 * kWSeg) + r * kWSeg;
+    const char* xb = smem + stage * STAGE + W_TILE + kw * X_TILE;
+    const int k_step = (s * KW + kw) * KS;
+    if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
+    qmm_static_for<SUB>([&](auto tc) {
+      constexpr int t = tc;
+      const int k_sub = k_step + t * 128;
+      if (kFull || k_sub < K) {
+        i32x4 wq0, wq1;
+        if constexpr (BITS == 8) {
+          wq0 = *(const i32x4*)(wb + (((8 * t + 2 * g) ^ r) * 16));
+          wq1 = *(const i32x4*)(wb + (((8 * t + 2 * g + 1) ^ r) * 16));
+        } else {
+          wq0 = *(const i32x4*)(wb + (((4 * t + g) ^ r) * 16));
+          wq1 = wq0;
         }
+        i32x4 xq[MT][XQ];
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          qmm_static_for<XQ>([&](auto qc) {
+            constexpr int q = qc;
+            xq[mt][q] = *(const i32x4*)(xb + (16 * mt + r) * XROW + (((XQ * 4 * t + XQ * g + q) ^ r) * 16));
+          });
+        });
+        if constexpr (kMfma) {
+          qmm_static_for<4>([&](auto jc) {
+            constexpr int j = jc;
+            i32x4 af;
+            if constexpr (BITS == 8) {
+              const i32x4 src = (j >> 1) ? wq1 : wq0;
+              af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
+            } else {
+              af = cvt_w4<XT>((uint32_t)wq0[j]);
+            }
+            qmm_static_for<MT>([&](auto mc) {
+              constexpr int mt = mc;
+              if constexpr (j & 1) accb[mt] = mfma16<XT>(af, xq[mt][j], accb[mt]);
+              else acc[mt] = mfma16<XT>(af, xq[mt][j], acc[mt]);
+              if constexpr (NEEDXS) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt][j], xs[mt]);
+            });
+          });
+        } else {
+          // f32 x: 16x16x4 f32 MFMA, one column per lane per instruction.
+          qmm_static_for<32>([&](auto kc) {
+            constexpr int kk = kc;  // 0..31 within the lane's columns
+            float wf;
+            if constexpr (BITS == 8) {
+              const i32x4 src = (kk >> 4) ? wq1 : wq0;
+              const uint32_t dw = (uint32_t)src[(kk >> 2) & 3];
+              wf = (float)(int8_t)(dw >> (8 * (kk & 3)));
+            } else {
+              // column kk = 8*word + P[nibble]: nibble = (c&1)*4 + (c>>1), c = kk % 8
+              const uint32_t dw = (uint32_t)wq0[kk >> 3];
+              constexpr int c = kk & 7, nib = (c & 1) * 4 + (c >> 1);
+              wf = (float)(int)((dw >> (4 * nib)) & 15u) - 8.0f;
+            }
+            qmm_static_for<MT>([&](auto mc) {
+              constexpr int mt = mc;
+              constexpr int xq_i = kk >> 2, xe_i = kk & 3;
+              const f32x4 xv4 = __builtin_bit_cast(f32x4, xq[mt][xq_i]);
+              const float xv = xv4[xe_i];
+              if constexpr (kk & 1) accb[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv, accb[mt], 0, 0, 0);
+              else acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv, acc[mt], 0, 0, 0);
+              if constexpr (NEEDXS) xs[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, xv, xs[mt], 0, 0, 0);
+            });
+          });
+        }
+        if constexpr (RED != kRedRaw) {
+          if (--block_left == 0) {
+            block_epilogue(k_sub / C);
+            block_left = sub_per_block;
+          }
+        }
+      }
+    });
+  };
+
+  // ---- main loop: registers hold loads of P steps ahead, LDS holds NS stages -----------
+  qmm_static_for<P>([&](auto pc) {
+    if (pc < my_steps) load_regs(pc, pc);
+  });
+  for (int s0 = 0; s0 < trips; s0 += 2) {
+    qmm_static_for<2>([&](auto hc) {
+      const int s = s0 + hc;
+      if (s < trips) {
+        constexpr int p = hc % P;
+        const int stage = NS == 2 ? (int)hc : 0;
+        if constexpr (NS == 1) {
+          if (s > 0) __syncthreads();  // the single stage is free again
+        }
+#ifndef QMM_SK_DBG
+#define QMM_SK_DBG 0
+#endif
+        if constexpr (!(QMM_SK_DBG & 2)) { if (s < my_steps) store_lds(qmm_const<p>{}, stage); }
+        if (s + P < my_steps) load_regs(qmm_const<p>{}, s + P);
+        if constexpr (!(QMM_SK_DBG & 4)) __syncthreads();
+        if constexpr (!(QMM_SK_DBG & 1)) {
+          if (s < my_steps) {
+            if (((s * KW + kw) + 1) * KS <= K) compute(qmm_const<1>{}, stage, s);
+            else compute(qmm_const<0>{}, stage, s);
+          }
+        }
+        if constexpr ((QMM_SK_DBG & 3) == 3) { qmm_static_for<8>([&](auto ic) { constexpr int i = ic; acc[0] += __builtin_bit_cast(f32x4, wreg[p][i]); }); qmm_static_for<XP>([&](auto ic) { constexpr int i = ic; acc[0] += __builtin_bit_cast(f32x4, xreg[p][i]); }); }
       }
     });
   }
 
-  if constexpr (PERCH) {
-    // Reduce raw partial sums over the waves.
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) red[wv][(rg * MT + mt) * 4 + v][lane] = acc[rg][mt][v];
-    if constexpr (NEEDXS) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) red[wv][kSlots + mt][lane] = xs[mt][0];
-    }
-  } else {
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          red[wv][(rg * MT + mt) * 4 + v][lane] = sacc[rg][mt][v];
-          if constexpr (HASZP) red[wv][kSlots + (rg * MT + mt) * 4 + v][lane] = zacc[rg][mt][v];
-        }
-  }
-  __syncthreads();
-
-  // Final epilogue: thread (wv, lane) finishes slots wv, wv + kWaves, ...
+  // ---- reduction over k-splits, final rounding, store ------------------------------------
   const int zpo_dt = qmm_promote(x_dt, a.zp_dt);
-  for (int slot = wv; slot < kSlots; slot += kWaves) {
-    int v = slot & 3, mt = (slot >> 2) % MT, rg = (slot >> 2) / MT;
-    int n = n_base + 16 * rg + 4 * g + v;
-    int m = 16 * mt + r;
-    float tot = 0.f, aux = 0.f;
+  if constexpr (KW > 1) {
+    __syncthreads();  // pipeline stages are dead: reuse LDS
+    float* red = (float*)smem;  // [KW][RW][slot][64]
+    constexpr int kSlots = RED == kRedRaw ? 4 * MT + (NEEDXS ? MT : 0) : (HASZP ? 8 * MT : 4 * MT);
+    float* mine = red + ((kw * RW + rw) * kSlots) * 64 + lane;
+    qmm_static_for<MT>([&](auto mc) {
+      constexpr int mt = mc;
+      qmm_static_for<4>([&](auto vc) {
+        constexpr int v = vc;
+        if constexpr (RED == kRedRaw) {
+          mine[(4 * mt + v) * 64] = acc[mt][v] + accb[mt][v];
+        } else {
+          mine[(4 * mt + v) * 64] = sacc[mt][v];
+          if constexpr (HASZP) mine[(4 * MT + 4 * mt + v) * 64] = zacc[mt][v];
+        }
+      });
+      if constexpr (RED == kRedRaw && NEEDXS) mine[(4 * MT + mt) * 64] = xs[mt][0];
+    });
+    __syncthreads();
+    if (kw != 0) return;
+    qmm_static_for<MT>([&](auto mc) {
+      constexpr int mt = mc;
+      qmm_static_for<4>([&](auto vc) {
+        constexpr int v = vc;
+        float t = 0.f, z = 0.f;
 #pragma unroll
-    for (int w2 = 0; w2 < kWaves; ++w2) tot += red[w2][slot][lane];
-    float o;
-    if constexpr (PERCH) {
-      if constexpr (NEEDXS) {
+        for (int k2 = 0; k2 < KW; ++k2) {
+          const float* other = red + ((k2 * RW + rw) * kSlots) * 64 + lane;
+          t += other[(4 * mt + v) * 64];
+          if constexpr (RED == kRedScaled && HASZP) z += other[(4 * MT + 4 * mt + v) * 64];
+        }
+        if constexpr (RED == kRedRaw) { acc[mt][v] = t; accb[mt][v] = 0.f; }
+        else { sacc[mt][v] = t; zacc[mt][v] = z; }
+      });
+      if constexpr (RED == kRedRaw && NEEDXS) {
+        float t = 0.f;
 #pragma unroll
-        for (int w2 = 0; w2 < kWaves; ++w2) aux += red[w2][kSlots + mt][lane];
+        for (int k2 = 0; k2 < KW; ++k2) t += (red + ((k2 * RW + rw) * kSlots) * 64 + lane)[(4 * MT + mt) * 64];
+        xs[mt] = f32x4{t, t, t, t};
       }
-      if (n >= N || m >= M) continue;
-      float p = qmm_round_dt(true_dot(tot, aux), x_dt);
-      o = qmm_round_dt(p * qmm_load(a.scale, n, a.scale_dt), a.out_dt);
+    });
+  }
+  if constexpr (RED == kRedRaw) block_epilogue(0);  // the single block ends here
+
+  qmm_static_for<MT>([&](auto mc) {
+    constexpr int mt = mc;
+    const int m = 16 * mt + r;
+    const int n = n_wave + 4 * g;
+    if (m < M && n < N) {
+      float o0 = qmm_round_dt(sacc[mt][0], a.out_dt), o1 = qmm_round_dt(sacc[mt][1], a.out_dt);
+      float o2 = qmm_round_dt(sacc[mt][2], a.out_dt), o3 = qmm_round_dt(sacc[mt][3], a.out_dt);
       if constexpr (HASZP) {
-        float z = qmm_round_dt(qmm_round_dt(aux, x_dt) * qmm_load(a.zp, n, a.zp_dt), zpo_dt);
-        o = qmm_round_dt(o - z, a.out_dt);
+        o0 = qmm_round_dt(o0 - qmm_round_dt(zacc[mt][0], zpo_dt), a.out_dt);
+        o1 = qmm_round_dt(o1 - qmm_round_dt(zacc[mt][1], zpo_dt), a.out_dt);
+        o2 = qmm_round_dt(o2 - qmm_round_dt(zacc[mt][2], zpo_dt), a.out_dt);
+        o3 = qmm_round_dt(o3 - qmm_round_dt(zacc[mt][3], zpo_dt), a.out_dt);
       }
-    } else {
-      if constexpr (HASZP) {
-#pragma unroll
-        for (int w2 = 0; w2 < kWaves; ++w2) aux += red[w2][kSlots + slot][lane];
+      const size_t idx = (size_t)m * N + n;
+      if ((N & 3) == 0) {  // 4 consecutive channels: one aligned 8- or 16-byte store
+        if (a.out_dt == XLA_AMD_DT_F32) {
+          *(f32x4*)((float*)a.out + idx) = f32x4{o0, o1, o2, o3};
+        } else {
+          const bool bf = a.out_dt == XLA_AMD_DT_BF16;
+          const uint32_t h0 = bf ? qmm_f32_to_bf16(o0) : qmm_f32_to_f16(o0);
+          const uint32_t h1 = bf ? qmm_f32_to_bf16(o1) : qmm_f32_to_f16(o1);
+          const uint32_t h2 = bf ? qmm_f32_to_bf16(o2) : qmm_f32_to_f16(o2);
+          const uint32_t h3 = bf ? qmm_f32_to_bf16(o3) : qmm_f32_to_f16(o3);
+          *(i32x2*)((uint16_t*)a.out + idx) = i32x2{(int)(h0 | (h1 << 16)), (int)(h2 | (h3 << 16))};
+        }
+      } else {
+        qmm_store(a.out, idx, o0, a.out_dt);
+        if (n + 1 < N) qmm_store(a.out, idx + 1, o1, a.out_dt);
+        if (n + 2 < N) qmm_store(a.out, idx + 2, o2, a.out_dt);
+        if (n + 3 < N) qmm_store(a.out, idx + 3, o3, a.out_dt);
       }
-      if (n >= N || m >= M) continue;
-      o = qmm_round_dt(tot, a.out_dt);
-      if constexpr (HASZP) o = qmm_round_dt(o - qmm_round_dt(aux, zpo_dt), a.out_dt);
     }
-    qmm_store(a.out, (int64_t)m * N + n, o, a.out_dt);
+  });
+}
+
+template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
+int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
+  using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
+  if constexpr (!Cfg::kFits) {
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: tile does not fit in LDS");
+  } else {
+    auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP>;
+    static thread_local bool attr_set = false;
+    if (!attr_set) {
+      int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 Cfg::LDS_BYTES), "weight_only_skinny hipFuncSetAttribute");
+      if (rc != XLA_AMD_QMM_OK) return rc;
+      attr_set = true;
+    }
+    const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWaves * 64), Cfg::LDS_BYTES, stream, a);
+    return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
 
-#ifndef QMM_SKINNY_RG
-#define QMM_SKINNY_RG 1
-#endif
-#ifndef QMM_SKINNY_D
-#define QMM_SKINNY_D 0
-#endif
-
-// Pipeline depth: as many iterations in flight as ~150 VGPRs of staging allow.
-constexpr int pipeline_depth(int xt, int mt) {
-  if (QMM_SKINNY_D > 0) return QMM_SKINNY_D;
-  if (xt == XLA_AMD_DT_F32) return mt <= 2 ? 2 : 1;
-  return mt == 1 ? 4 : (mt == 2 ? 3 : 2);
+template <int XT, int BITS, int MT, int KW, int RED>
+int launch_zp(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
+  return haszp ? launch_kernel<XT, BITS, MT, KW, RED, true>(a, stream)
+               : launch_kernel<XT, BITS, MT, KW, RED, false>(a, stream);
 }
 
-template <int XT, int BITS, int MT, bool PERCH, bool HASZP>
-int launch_rg(const SkinnyArgs& a, hipStream_t stream) {
-  constexpr int RG = QMM_SKINNY_RG;
-  constexpr int D = pipeline_depth(XT, MT);
-  unsigned blocks = (unsigned)((a.N + 16 * RG - 1) / (16 * RG));
-  hipLaunchKernelGGL((qmm_skinny_kernel<XT, BITS, MT, RG, D, PERCH, HASZP>), dim3(blocks),
-                     dim3(kWaves * 64), 0, stream, a);
-  return QMM_CHECK_LAUNCH("weight_only_skinny launch");
-}
-
+// k-splits per workgroup: as few as keep >= ~200 workgroups, and only where the
+// reduction is defined (per-channel, or whole quantization blocks per step) and
+// the wider x tile still fits in LDS.
 template <int XT, int BITS, int MT>
-int launch_mode(const SkinnyArgs& a, bool perch, bool haszp, hipStream_t stream) {
-  if (perch) return haszp ? launch_rg<XT, BITS, MT, true, true>(a, stream) : launch_rg<XT, BITS, MT, true, false>(a, stream);
-  return haszp ? launch_rg<XT, BITS, MT, false, true>(a, stream) : launch_rg<XT, BITS, MT, false, false>(a, stream);
+int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
+  constexpr int KS = BITS == 8 ? kWSeg : 2 * kWSeg;
+  const bool perch = a.C == a.K;
+  const bool can_split = perch || (KS % a.C == 0);
+  const int steps = (a.K + KS - 1) / KS;
+  int kw = 1;
+  if (can_split) {
+    if (a.N < 200 * 64 && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
+    if (a.N < 200 * 32 && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
+  }
+  if (kw == 1) return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
+                            : launch_zp<XT, BITS, MT, 1, kRedNone>(a, haszp, stream);
+  if (kw == 2) return perch ? launch_zp<XT, BITS, MT, 2, kRedRaw>(a, haszp, stream)
+                            : launch_zp<XT, BITS, MT, 2, kRedScaled>(a, haszp, stream);
+  return perch ? launch_zp<XT, BITS, MT, 4, kRedRaw>(a, haszp, stream)
+               : launch_zp<XT, BITS, MT, 4, kRedScaled>(a, haszp, stream);
 }
 
 template <int XT, int BITS>
-int launch_mt(const SkinnyArgs& a, bool perch, bool haszp, hipStream_t stream) {
-  if (a.M <= 16) return launch_mode<XT, BITS, 1>(a, perch, haszp, stream);
-  if (a.M <= 32) return launch_mode<XT, BITS, 2>(a, perch, haszp, stream);
-  return launch_mode<XT, BITS, 4>(a, perch, haszp, stream);
+int launch_mt(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
+  if constexpr (XT != XLA_AMD_DT_F32) {
+    if (a.M > 16) return launch_split<XT, BITS, 2>(a, haszp, stream);
+  }
+  return launch_split<XT, BITS, 1>(a, haszp, stream);
 }
 
 template <int XT>
-int launch_bits(const SkinnyArgs& a, int bits, bool perch, bool haszp, hipStream_t stream) {
-  return bits == 8 ? launch_mt<XT, 8>(a, perch, haszp, stream) : launch_mt<XT, 4>(a, perch, haszp, stream);
+int launch_bits(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream) {
+  return bits == 8 ? launch_mt<XT, 8>(a, haszp, stream) : launch_mt<XT, 4>(a, haszp, stream);
 }
 
 }  // namespace
@@ -412,31 +553,32 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packe
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: bad dtype enum");
   if (out_dt != qmm_promote(x_dt, scale_dt))
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: out dtype must be promote(x, scale)");
-  if (K % kKIter != 0 || C % kKIter != 0)
-    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: K=%lld and C=%lld must be multiples of %d",
-                    (long long)K, (long long)C, kKIter);
-  if (N > (1 << 30) || K > (1 << 30) || M > (1 << 30))
+  if (K % 128 != 0 || C % 128 != 0)
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: K=%lld and C=%lld must be multiples of 128",
+                    (long long)K, (long long)C);
+  if (N > (1 << 30) || K > (1 << 24) || M > (1 << 30))
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: dimension too large");
   if (((uintptr_t)x | (uintptr_t)w_packed) & 15)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: x and w must be 16-byte aligned");
+  if (((uintptr_t)out & 15) && (N & 3) == 0)
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: out must be 16-byte aligned");
   if (M == 0) return XLA_AMD_QMM_OK;
-  const bool perch = (C == K);
   const int xsz = qmm_dt_size(x_dt), osz = qmm_dt_size(out_dt);
-  // Up to 64 rows of x per pass over the weight.
-  for (int64_t m0 = 0; m0 < M; m0 += 64) {
+  const int pass = x_dt == XLA_AMD_DT_F32 ? 16 : 32;  // rows of x per pass over the weight
+  for (int64_t m0 = 0; m0 < M; m0 += pass) {
     SkinnyArgs a;
     a.x = (const char*)x + (size_t)m0 * K * xsz;
     a.w = (const uint8_t*)w_packed;
     a.scale = scale;
     a.zp = zp;
     a.out = (char*)out + (size_t)m0 * N * osz;
-    a.M = (int)((M - m0) < 64 ? (M - m0) : 64);
+    a.M = (int)((M - m0) < pass ? (M - m0) : pass);
     a.N = (int)N; a.K = (int)K; a.C = (int)C;
     a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.out_dt = out_dt;
     int rc;
-    if (x_dt == XLA_AMD_DT_BF16) rc = launch_bits<XLA_AMD_DT_BF16>(a, bits, perch, zp != nullptr, (hipStream_t)stream);
-    else if (x_dt == XLA_AMD_DT_F16) rc = launch_bits<XLA_AMD_DT_F16>(a, bits, perch, zp != nullptr, (hipStream_t)stream);
-    else rc = launch_bits<XLA_AMD_DT_F32>(a, bits, perch, zp != nullptr, (hipStream_t)stream);
+    if (x_dt == XLA_AMD_DT_BF16) rc = launch_bits<XLA_AMD_DT_BF16>(a, bits, zp != nullptr, (hipStream_t)stream);
+    else if (x_dt == XLA_AMD_DT_F16) rc = launch_bits<XLA_AMD_DT_F16>(a, bits, zp != nullptr, (hipStream_t)stream);
+    else rc = launch_bits<XLA_AMD_DT_F32>(a, bits, zp != nullptr, (hipStream_t)stream);
     if (rc != XLA_AMD_QMM_OK) return rc;
   }
   return XLA_AMD_QMM_OK;
