@@ -39,6 +39,15 @@ typedef int i32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also makes
+// every wave wait for its outstanding *global* loads (its fence covers all
+// address spaces), which would drain the prefetch pipeline at every step.
+__device__ __forceinline__ void qmm_lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ float qmm_bf16_to_f32(uint16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }

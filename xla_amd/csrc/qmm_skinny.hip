@@ -25,6 +25,11 @@
 // in lane (j + 16*(i/4)), register i%4: channel 4g + v, x row r.
 #include "qmm_common.h"
 
+#ifdef QMM_SK_NONT
+#define QMM_SK_LOAD(p) (*(p))
+#else
+#define QMM_SK_LOAD(p) __builtin_nontemporal_load(p)
+#endif
 namespace {
 
 constexpr int kWaves = 4;
@@ -129,7 +134,10 @@ struct SkinnyCfg {
   static constexpr int STAGE = W_TILE + KW * X_TILE;
   static constexpr int NS = 2 * STAGE <= kLdsLimit ? 2 : 1;  // LDS stages
   static constexpr int XP = X_TILE / 1024 / RW;              // 1 KB x loads per wave per step
-  static constexpr int P = (32 + 4 * XP) <= 64 ? 2 : 1;      // steps of loads in flight (register ring)
+#ifndef QMM_SK_P
+#define QMM_SK_P 2
+#endif
+  static constexpr int P = ((32 + 4 * XP) <= 64 && QMM_SK_P == 2) ? 2 : 1;      // steps of loads in flight (register ring)
   static constexpr int LDS_BYTES = NS * STAGE;
   static constexpr bool kFits = STAGE <= kLdsLimit;
   static_assert((X_TILE / 1024) % RW == 0, "x tile must split evenly over the waves of a k-split");
@@ -194,13 +202,15 @@ qmm_skinny_kernel(SkinnyArgs a) {
   i32x4 xreg[P][XP];
   auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {  // s: this wave's s-th step
     constexpr int p = pc;
-    const int gs = s * KW + kw;  // global step
+    // global step; steps past the end (issued only to keep the number of
+    // outstanding loads the same on every path) re-read the last real step
+    const int gs = min(s * KW + kw, steps_total - 1);
     const uint8_t* const wp = w_base + (size_t)gs * kWSeg;
     const char* const xp = x_base + (size_t)gs * XROW;
     if ((gs + 1) * KS <= K) {  // whole step inside K: no per-lane conditions
       qmm_static_for<8>([&](auto ic) {
         constexpr int i = ic;
-        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
+        wreg[p][i] = QMM_SK_LOAD((const i32x4*)(wp + w_off[i]));
       });
       qmm_static_for<XP>([&](auto jc) {
         constexpr int j = jc;
@@ -212,15 +222,17 @@ qmm_skinny_kernel(SkinnyArgs a) {
       const int w_left = row_bytes - gs * kWSeg, x_left = K * XB - gs * XROW;
       qmm_static_for<8>([&](auto ic) {
         constexpr int i = ic;
-        const uint32_t back = (uint32_t)max(w_chunk * 16 + 16 - w_left, 0);
-        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + (w_off[i] - back)));
+        // w_left >= 64 here, so 0 <= back <= w_chunk * 16 <= w_off[i]
+        const int back = max(w_chunk * 16 + 16 - w_left, 0);
+        wreg[p][i] = QMM_SK_LOAD((const i32x4*)(wp + ((int64_t)w_off[i] - back)));
       });
       qmm_static_for<XP>([&](auto jc) {
         constexpr int j = jc;
         constexpr int kPiecesPerRow = XROW / 1024;
         const int col = (((rw * XP + j) % kPiecesPerRow) * 64 + lane) * 16;
-        const uint32_t back = (uint32_t)max(col + 16 - x_left, 0);
-        xreg[p][j] = *(const i32x4*)(xp + (x_off[j] - back));
+        // x_left >= 256 here, so 0 <= back <= col <= x_off[j]
+        const int back = max(col + 16 - x_left, 0);
+        xreg[p][j] = *(const i32x4*)(xp + ((int64_t)x_off[j] - back));
       });
     }
   };
@@ -367,31 +379,32 @@ qmm_skinny_kernel(SkinnyArgs a) {
   };
 
   // ---- main loop: registers hold loads of P steps ahead, LDS holds NS stages -----------
-  qmm_static_for<P>([&](auto pc) {
-    if (pc < my_steps) load_regs(pc, pc);
-  });
-  for (int s0 = 0; s0 < trips; s0 += 2) {
-    qmm_static_for<2>([&](auto hc) {
+  // Loads are issued unconditionally, also for steps past the end (those take
+  // the clamped path and are never consumed): a load that is issued on some
+  // paths only would force the compiler to wait for *all* outstanding loads
+  // wherever it needs one of them.
+  qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
+#ifndef QMM_SK_UNROLL
+#define QMM_SK_UNROLL 2
+#endif
+  constexpr int kUnroll = QMM_SK_UNROLL;  // steps per loop trip: the compiler's wait-count bookkeeping is exact
+                              // inside straight-line code and conservative across the back edge
+  for (int s0 = 0; s0 < trips; s0 += kUnroll) {
+    qmm_static_for<kUnroll>([&](auto hc) {
       const int s = s0 + hc;
       if (s < trips) {
         constexpr int p = hc % P;
-        const int stage = NS == 2 ? (int)hc : 0;
+        const int stage = NS == 2 ? (int)(hc % 2) : 0;
         if constexpr (NS == 1) {
-          if (s > 0) __syncthreads();  // the single stage is free again
+          if (s > 0) qmm_lds_barrier();  // the single stage is free again
         }
-#ifndef QMM_SK_DBG
-#define QMM_SK_DBG 0
-#endif
-        if constexpr (!(QMM_SK_DBG & 2)) { if (s < my_steps) store_lds(qmm_const<p>{}, stage); }
-        if (s + P < my_steps) load_regs(qmm_const<p>{}, s + P);
-        if constexpr (!(QMM_SK_DBG & 4)) __syncthreads();
-        if constexpr (!(QMM_SK_DBG & 1)) {
-          if (s < my_steps) {
-            if (((s * KW + kw) + 1) * KS <= K) compute(qmm_const<1>{}, stage, s);
-            else compute(qmm_const<0>{}, stage, s);
-          }
+        if (s < my_steps) store_lds(qmm_const<p>{}, stage);
+        load_regs(qmm_const<p>{}, s + P);
+        qmm_lds_barrier();
+        if (s < my_steps) {
+          if (((s * KW + kw) + 1) * KS <= K) compute(qmm_const<1>{}, stage, s);
+          else compute(qmm_const<0>{}, stage, s);
         }
-        if constexpr ((QMM_SK_DBG & 3) == 3) { qmm_static_for<8>([&](auto ic) { constexpr int i = ic; acc[0] += __builtin_bit_cast(f32x4, wreg[p][i]); }); qmm_static_for<XP>([&](auto ic) { constexpr int i = ic; acc[0] += __builtin_bit_cast(f32x4, xreg[p][i]); }); }
       }
     });
   }
@@ -477,6 +490,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
   });
 }
 
+#ifdef QMM_SK_PROBE
+template __global__ void qmm_skinny_kernel<XLA_AMD_DT_BF16, 8, 1, 1, kRedRaw, false>(SkinnyArgs);
+}  // namespace
+#else
 template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
 int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
   using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
@@ -583,3 +600,4 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packe
   }
   return XLA_AMD_QMM_OK;
 }
+#endif  // QMM_SK_PROBE
