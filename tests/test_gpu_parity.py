@@ -229,3 +229,108 @@ def test_quantized_matmul_int8_op(ops):
     out = torch.ops.xla.quantized_matmul_int8(*dev(x, w, s), quantize_activation=True)
     assert out.dtype == torch.bfloat16
     check(out, exp, "quantized_matmul_int8")
+
+
+# ---- committed golden fixtures through the HIP path ----------------------------------------
+import json
+import os
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "quantized_matmul_golden.json")))
+
+
+def _bf16_from_bits(bits):
+  return torch.tensor(np.asarray(bits, dtype=np.uint16).astype(np.int32)).to(torch.int16).view(torch.bfloat16)
+
+
+def test_golden_hand_cases(ops):
+  g = GOLD["hand_per_channel"]
+  x, w = torch.tensor(g["x"]), torch.tensor(g["w"], dtype=torch.int8)
+  s, z = torch.tensor(g["scale"]), torch.tensor(g["zp"])
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, s)).cpu(), torch.tensor(g["expect"]))
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, s, z)).cpu(), torch.tensor(g["expect_zp"]))
+  g = GOLD["hand_blockwise"]
+  x, w = torch.tensor(g["x"]), torch.tensor(g["w"], dtype=torch.int8)
+  s, z = torch.tensor(g["scale"]), torch.tensor(g["zp"])
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, s), block_size=2).cpu(), torch.tensor(g["expect"]))
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=2).cpu(), torch.tensor(g["expect_zp"]))
+
+
+def test_golden_overflow_band_and_w8a8(ops):
+  g = GOLD["bf16_overflow_band"]
+  x = _bf16_from_bits(g["maxima_bits"]).reshape(-1, 1).contiguous()
+  for policy in ("saturate", "wrap"):
+    q, s, _ = ops.quantize_per_token_gpu(x.cuda(), overflow=policy)
+    assert q.cpu().flatten().tolist() == g["q_" + policy]
+    assert torch.equal(s.cpu().flatten(), _bf16_from_bits(g["scale_bits"]))
+  g = GOLD["w8a8_seeded"]
+  x = _bf16_from_bits(np.asarray(g["x_bits"])).reshape(4, 256).contiguous()
+  w = torch.tensor(g["w"], dtype=torch.int8)
+  q, s, _ = ops.quantize_per_token_gpu(x.cuda())
+  assert torch.equal(q.cpu().long(), torch.tensor(g["x_q"]))
+  assert torch.equal(s.cpu().flatten(), _bf16_from_bits(g["x_scale_bits"]))
+  _, acc = ops.w8a8_gemm_gpu(q, w.cuda(), s, torch.ones(64).cuda(), None, None, cvt_dtype=torch.float32,
+                             mid_dtype=torch.float32, out_dtype=torch.float32, want_acc=True)
+  assert torch.equal(acc.cpu().long(), torch.tensor(g["acc"]))
+
+
+def test_golden_dot_general_and_int4_pack(ops):
+  from xla_amd import _lib
+  g = GOLD["dot_general_int32"]
+  a, b = torch.tensor(g["a"], dtype=torch.int8), torch.tensor(g["b"], dtype=torch.int8)
+  for i in range(a.shape[0]):
+    _, acc = ops.w8a8_gemm_gpu(a[i].contiguous().cuda(), b[i].T.contiguous().cuda(), torch.ones(3, 1).cuda(),
+                               torch.ones(5).cuda(), None, None, cvt_dtype=torch.float32,
+                               mid_dtype=torch.float32, out_dtype=torch.float32, want_acc=True)
+    assert torch.equal(acc.cpu().long(), torch.tensor(g["expect"][i]))
+  rows = GOLD["int4_pack"]
+  w = torch.tensor([r["values"] for r in rows], dtype=torch.int8)  # [16, 8]
+  for layout, src in ((_lib.W_NK, w), (_lib.W_SCN, w.T.reshape(1, 8, 16).contiguous())):
+    packed = ops._packed_weight(src.cuda(), 4, layout).cpu().numpy().view(np.uint32)
+    assert packed.tolist() == [r["word"] for r in rows]
+
+
+def test_w8a8_tiles_and_tails(ops):
+  # every workgroup tile the kernel offers, on shapes with M/N/K tails
+  for bm in (64, 128, 256):
+    for (m, n, k) in [(bm + 3, 2 * bm + 5, 144), (17, 33, 64), (bm, bm, 4096)]:
+      g = cases.gen(bm + m + n)
+      xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+      w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+      _, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), torch.ones(m, 1).cuda(), torch.ones(n).cuda(), None, None,
+                                 cvt_dtype=torch.float32, mid_dtype=torch.float32, out_dtype=torch.float32,
+                                 want_acc=True, block_m=bm, block_n=bm)
+      ref = torch.from_numpy(xq.numpy().astype(np.int64) @ w.numpy().astype(np.int64).T)
+      assert torch.equal(acc.cpu().long(), ref), (bm, m, n, k)
+
+
+def test_skinny_k_splits_and_long_k(ops):
+  # small N takes k-split workgroups; K = 14336 is the down projection; M > 32 takes two passes
+  for (m, n, k, xdt) in [(16, 256, 4096, torch.bfloat16), (5, 4096, 14336, torch.bfloat16), (40, 1024, 1024, torch.bfloat16),
+                         (8, 2048, 2048, torch.float32), (16, 4096, 640, torch.float16)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=n + k)
+    exp = oracle.quantized_matmul(x, w, s)
+    out = torch.ops.xla.quantized_matmul(*dev(x, w, s))
+    check(out, exp, f"skinny {m, n, k, xdt}")
+  # blockwise with blocks wider than a step (C = 1024) and K tail of the last step
+  x, w, s, z, _ = cases.blockwise(16, 512, 3072, 1024, 8, torch.bfloat16, symmetric=False, seed=9)
+  check(torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=1024),
+        oracle.quantized_matmul(x, w, s, z, block_size=1024), "blockwise C=1024")
+  x, w, s, z, _ = cases.blockwise(16, 512, 640, 128, 4, torch.bfloat16, symmetric=False, seed=10)
+  check(torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=128, int4_weight=True),
+        oracle.quantized_matmul(x, w, s, z, block_size=128), "blockwise int4 K=640")
+
+
+def test_module_and_state_dict_on_gpu(ops):
+  from xla_amd.quantization import quantize_linear
+  lin = torch.nn.Linear(256, 64, bias=False)
+  x = torch.randn(3, 7, 256)
+  for kw in (dict(n_bits=8), dict(n_bits=8, symmetric=False), dict(n_bits=4, block_size=128, symmetric=False),
+             dict(n_bits=8, quantize_activation=True)):
+    q = quantize_linear(lin, **kw)
+    exp = oracle.quantized_matmul(x, q.weight, q.weight_scaler, q.zero_point, block_size=q.block_size,
+                                  quantize_activation=q.quantize_activation)
+    qd = q.cuda()
+    out = qd(x.cuda())
+    assert out.shape == (3, 7, 64)
+    check(out, exp, f"module {kw}")
+    assert qd.weight.is_cuda and set(qd.state_dict()) >= {"weight", "weight_scaler"}

@@ -1,0 +1,183 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what
+include/xla_amd_qmm.h declares, the dispatcher, operator registration, argument
+checks with the reference's messages, the module and the quantizer utilities."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from oracle import quantized_matmul_oracle as oracle
+from tests import cases
+from xla_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def qmm():
+  import xla_amd.experimental.custom_kernel  # noqa: F401
+  import xla_amd.experimental.xla_quantized_matmul as m
+  return m
+
+
+def declared_functions():
+  text = open(os.path.join(ROOT, "include", "xla_amd_qmm.h")).read()
+  text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+  return sorted(set(re.findall(r"\b(xla_amd_qmm_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+  lib = _lib.load()
+  names = declared_functions()
+  assert len(names) >= 10
+  for n in names:
+    assert hasattr(lib, n), f"{n} declared in the header but not exported"
+  assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
+  assert lib.xla_amd_qmm_abi_version() == 1
+
+
+def test_header_cites_reference_for_each_entry_point():
+  text = open(os.path.join(ROOT, "include", "xla_amd_qmm.h")).read()
+  for key in ("xla_quantized_matmul.py", "custom_kernel.py", "dot_general.cpp", "cast_int4.cpp",
+              "quantized_matmul_kernel.py"):
+    assert key in text
+
+
+def test_dispatcher_regimes():
+  lib = _lib.load()
+  d = lib.xla_amd_qmm_dispatch
+  assert d(16, 14336, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA
+  assert d(1, 4096, 4096, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA
+  assert d(3, 8, 5, 5, 8, _lib.DT_F32, 0) == _lib.KERNEL_GENERIC
+  assert d(3, 8, 6, 2, 8, _lib.DT_F32, 0) == _lib.KERNEL_GENERIC
+  assert d(2048, 14336, 4096, 4096, 8, _lib.DT_BF16, 1) == _lib.KERNEL_W8A8_MFMA
+  assert d(3, 8, 5, 5, 8, _lib.DT_F32, 1) == _lib.KERNEL_W8A8_GENERIC
+  tile = (ctypes.c_int32 * 3)()
+  assert lib.xla_amd_qmm_w8a8_tile(2048, 14336, 4096, tile) == 0
+  assert list(tile) == [256, 256, 128]
+  assert lib.xla_amd_qmm_w8a8_tile(64, 64, 64, tile) == 0 and list(tile)[:2] == [64, 64]
+
+
+def test_error_codes_without_gpu():
+  lib = _lib.load()
+  assert lib.xla_amd_qmm_packed_bytes(8, 64, 8) == 512
+  assert lib.xla_amd_qmm_packed_bytes(8, 64, 4) == 256
+  assert lib.xla_amd_qmm_packed_bytes(8, 5, 4) == 0
+  rc = lib.xla_amd_qmm_weight_only_skinny(None, None, None, None, None, 1, 1, 128, 128, 8, 1, 1, 1, 1, None)
+  assert rc == _lib.EINVAL and b"null" in lib.xla_amd_qmm_last_error()
+  rc = lib.xla_amd_qmm_quantize_per_token(None, None, None, None, 1, 1, 0, 0, 0, None)
+  assert rc == _lib.EINVAL
+  rc = lib.xla_amd_qmm_w8a8_gemm(None, None, None, None, None, None, None, None, 1, 1, 16, 0, 0, 0, 0, 0, 0, 0, 0, 0, None)
+  assert rc == _lib.EINVAL
+  with pytest.raises(RuntimeError, match="failed"):
+    _lib.check(rc, "w8a8_gemm")
+
+
+def test_ops_are_registered_with_reference_schemas(qmm):
+  s = str(torch.ops.xla.quantized_matmul.default._schema)
+  assert s == ("xla::quantized_matmul(Tensor x, Tensor w, Tensor scale, Tensor? zero_point=None, int? block_size=-1, "
+               "bool? int4_weight=False, bool? quantize_activation=False) -> Tensor")
+  s8 = str(torch.ops.xla.quantized_matmul_int8.default._schema)
+  assert s8.startswith("xla::quantized_matmul_int8(Tensor x, Tensor w, Tensor scalar, Tensor? zero_point=None, "
+                       "Tensor? quant_block_size=None, bool quantize_activation=False, int? batch_block_size=None")
+
+
+def test_cpu_tensors_take_the_eager_formulation(qmm):
+  x, w, s, _ = cases.per_channel_int8(4, 16, 32, torch.float32, torch.float32, seed=1)
+  z = torch.randn(16, generator=cases.gen(2)) * 0.01
+  assert torch.equal(torch.ops.xla.quantized_matmul(x, w, s, z), oracle.quantized_matmul(x, w, s, z))
+  xb, wb, sb, zb, _ = cases.blockwise(3, 8, 32, 8, 8, torch.float32, seed=3)
+  assert torch.equal(torch.ops.xla.quantized_matmul(xb, wb, sb, zb, block_size=8),
+                     oracle.quantized_matmul(xb, wb, sb, zb, block_size=8))
+  out = torch.ops.xla.quantized_matmul(x, w, s, quantize_activation=True)
+  assert torch.equal(out, oracle.quantized_matmul(x, w, s, quantize_activation=True, overflow="wrap"))
+
+
+def test_meta_tensors(qmm):
+  x = torch.empty(2, 3, 64, device="meta", dtype=torch.bfloat16)
+  w = torch.empty(32, 64, device="meta", dtype=torch.int8)
+  s = torch.empty(32, device="meta", dtype=torch.float32)
+  assert torch.ops.xla.quantized_matmul(x, w, s).shape == (2, 3, 32)
+  assert torch.ops.xla.quantized_matmul(x, w, s).dtype == torch.float32
+  assert torch.ops.xla.quantized_matmul(x, w, s.bfloat16(), quantize_activation=True).dtype == torch.bfloat16
+  x2 = torch.empty(10, 20, device="meta", dtype=torch.bfloat16)
+  w2 = torch.empty(30, 20, device="meta", dtype=torch.int8)
+  r = torch.ops.xla.quantized_matmul_int8(x2, w2, torch.empty(30, device="meta"), quantize_activation=True)
+  assert r.shape == (10, 30) and r.dtype == torch.bfloat16  # test/test_pallas.py:1030-1045
+
+
+def test_argument_checks_use_the_reference_messages(qmm):
+  x = torch.randn(3, 5)
+  w = torch.randint(-8, 8, (8, 5), dtype=torch.int8)
+  s = torch.rand(8)
+  with pytest.raises(AssertionError, match="Weight dtype is expected to be torch.int8"):
+    torch.ops.xla.quantized_matmul(x, w.float(), s)
+  with pytest.raises(AssertionError, match=r"Weight shape is expected to be \[output_dim, input_dim\]"):
+    torch.ops.xla.quantized_matmul(torch.randn(3, 6), w, s)
+  with pytest.raises(AssertionError, match="weight scaler shape is expect to be"):
+    torch.ops.xla.quantized_matmul(x, w, torch.rand(8, 1))
+  wb = torch.randint(-8, 8, (3, 2, 8), dtype=torch.int8)
+  with pytest.raises(AssertionError, match="Blockwise quantization does not support activation quantization"):
+    torch.ops.xla.quantized_matmul(torch.randn(3, 6), wb, torch.rand(3, 8), block_size=2, quantize_activation=True)
+  with pytest.raises(AssertionError, match="Weight tensor is expected to be 3D"):
+    torch.ops.xla.quantized_matmul(torch.randn(3, 6), torch.zeros(8, 6, dtype=torch.int8), torch.rand(3, 8), block_size=2)
+  with pytest.raises(AssertionError, match="input_dim should be divisible by block_size"):
+    torch.ops.xla.quantized_matmul(torch.randn(3, 7), wb, torch.rand(3, 8), block_size=2)
+
+
+def test_module_matches_reference_layout(qmm):
+  m = qmm.XlaQuantizedLinear(6, 8)
+  assert sorted(m.state_dict()) == ["weight", "weight_scaler", "zero_point"]
+  assert m.weight.dtype == torch.int8 and tuple(m.weight.shape) == (8, 6)
+  assert sorted(qmm.XlaQuantizedLinear(6, 8, is_symmetric=True).state_dict()) == ["weight", "weight_scaler"]
+  mb = qmm.XlaQuantizedLinear(6, 8, block_size=2)
+  assert tuple(mb.weight.shape) == (8, 6)  # 2-D until load_quantized_weight swaps it (as in the reference)
+  wb = torch.randint(-8, 8, (3, 2, 8), dtype=torch.int8)
+  mb.load_quantized_weight(wb, torch.rand(3, 8), torch.rand(3, 8))
+  assert tuple(mb.weight.shape) == (3, 2, 8)
+  with pytest.raises(AssertionError):
+    mb.load_quantized_weight(torch.zeros(8, 6, dtype=torch.int8), torch.rand(3, 8))
+  x = torch.randn(4, 6)
+  assert torch.equal(mb(x), oracle.quantized_matmul(x, mb.weight, mb.weight_scaler, mb.zero_point, block_size=2))
+
+
+def test_rtn_quantizer_and_module_swap(qmm):
+  from xla_amd.quantization import quantize_weight_rtn, replace_linear_with_quantized
+  g = cases.gen(5)
+  w_fp = torch.randn(16, 64, generator=g) * 0.02
+  for bits, block, sym in [(8, -1, True), (8, -1, False), (4, 16, False), (4, 16, True), (8, 32, False)]:
+    w, s, z = quantize_weight_rtn(w_fp, bits, block, sym)
+    qmin, qmax = -2**(bits - 1), 2**(bits - 1) - 1
+    assert w.dtype == torch.int8 and w.min() >= qmin and w.max() <= qmax
+    if block == -1:
+      assert tuple(w.shape) == (16, 64) and tuple(s.shape) == (16,)
+      deq = w.float() * s[:, None] - (0 if z is None else z[:, None])
+    else:
+      assert tuple(w.shape) == (64 // block, block, 16) and tuple(s.shape) == (64 // block, 16)
+      deq = (w.float() * s[:, None, :] - (0 if z is None else z[:, None, :])).reshape(64, 16).T
+    assert (deq - w_fp).abs().max() <= s.max() * 0.5 + 1e-6  # RTN error is at most half a step
+  net = torch.nn.Sequential(torch.nn.Linear(64, 32, bias=False), torch.nn.ReLU(), torch.nn.Linear(32, 8, bias=True))
+  x = torch.randn(5, 64, generator=g)
+  ref = net(x)
+  replace_linear_with_quantized(net, n_bits=8)
+  assert isinstance(net[0], qmm.XlaQuantizedLinear) and isinstance(net[2], torch.nn.Linear)
+  assert torch.allclose(net(x), ref, atol=0.05)
+
+
+def test_tuned_block_table(qmm):
+  from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import TUNED_BLOCK_SIZES, get_tuned_block_sizes
+  key0 = next(iter(TUNED_BLOCK_SIZES))
+  arch, bs, n_out, n_in, dt, qa = key0
+  assert get_tuned_block_sizes(TUNED_BLOCK_SIZES, bs, n_out, n_in, dt, qa, arch=arch) == TUNED_BLOCK_SIZES[key0]
+  assert get_tuned_block_sizes(TUNED_BLOCK_SIZES, 7, 9, 11, "bfloat16", True, arch=arch) == (None, None, None)
+  assert TUNED_BLOCK_SIZES[("gfx950", 2048, 14336, 4096, "bfloat16", True)] == (256, 256, 128)
+
+
+def test_product_does_not_import_the_oracle():
+  for dirpath, _, files in os.walk(os.path.join(ROOT, "xla_amd")):
+    for f in files:
+      if f.endswith((".py", ".hip", ".h", ".cpp")):
+        text = open(os.path.join(dirpath, f)).read()
+        assert "oracle" not in text.lower().replace("no fallback", ""), f"{f} mentions the oracle"
