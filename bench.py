@@ -30,6 +30,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA (5.0 POP/s)
 
 N_OUT, K_IN = 14336, 4096
+TRAFFIC_BYTES_PER_LAUNCH = 68.9e6  # decode GEMV M=16, see profiles/skinny_gemv_cfg2_m16_hbm_traffic.md
 
 
 def gemv_bytes(m, n, k, w_bytes_per_elem=1.0, x_b=2, s_b=2, out_b=2, n_scale_rows=1, zp=False):
@@ -46,6 +47,8 @@ def main():
   ap.add_argument("--no-graph", action="store_true", help="time eager calls instead of a HIP graph replay")
   ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--calibrate-copy", action="store_true",
+                  help="also run a plain 256 MiB device copy (known traffic, for scaling rocprof byte counters)")
   args = ap.parse_args()
   if args.gpus != 1:
     print("bench.py: this build measures one GPU; --gpus must be 1 (the kernels are not sharded, "
@@ -99,6 +102,14 @@ def main():
 
   use_graph = not args.no_graph
 
+  if args.calibrate_copy:
+    src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(4):
+      torch.add(src, 1, out=dst)  # elementwise kernel: 256 MiB read + 256 MiB written per launch
+    torch.cuda.synchronize()
+    del src, dst
+
   # ---- headline: decode GEMV, M = 16, rotating (cold) weights -----------------
   x16, w_cpu, s_cpu, _ = cases.per_channel_int8(16, N_OUT, K_IN, torch.bfloat16, torch.bfloat16, seed=2)
   n_rot = 12  # 12 x 58.7 MB = 704 MB > 512 MB
@@ -140,7 +151,10 @@ def main():
           "peak": HBM_PEAK_GBPS,
           "unit": "GB/s",
           "frac": round(achieved / HBM_PEAK_GBPS, 4),
-          "traffic": None,
+          # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from an
+          # elementwise kernel of known size); it is a profile result, not re-measured by this script
+          "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+          "traffic_source": "profiles/skinny_gemv_cfg2_m16_hbm_traffic.md",
           "kernel": "qmm_skinny_kernel<bf16, int8, MT=1>",
           "avg_launch_us": round(ev_ms * 1e3, 3),
       },
