@@ -75,37 +75,61 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int K = g.K;
 
-  // Global source of this thread's chunks (row clamped into the matrix).
+  // Global -> LDS copies bypass registers (global_load_lds_dwordx4): a wave
+  // instruction writes 64 x 16 bytes to consecutive LDS addresses (lane l at
+  // base + 16 l), i.e. 8 rows x 8 chunks of a stage.  The XOR swizzle of the
+  // LDS layout is therefore applied on the source side: LDS slot (row, c')
+  // receives global chunk c' ^ (row/2 % 8) of that row.  Rows are clamped
+  // into the matrix; chunks past K are zero-filled with a plain LDS store.
   const int8_t* ga[A_CH];
   const int8_t* gb[B_CH];
-  int lds_a[A_CH], lds_b[B_CH];
-  const int ck = tid & 7;  // chunk within the 128-byte row segment
-#pragma unroll
-  for (int i = 0; i < A_CH; ++i) {
-    int row = (i * T + tid) >> 3;
-    ga[i] = g.a + (size_t)min(m0 + row, g.M - 1) * K + ck * 16;
-    lds_a[i] = row * kBK + swz(row, ck) * 16;
-  }
-#pragma unroll
-  for (int i = 0; i < B_CH; ++i) {
-    int row = (i * T + tid) >> 3;
-    gb[i] = g.b + (size_t)min(n0 + row, g.N - 1) * K + ck * 16;
-    lds_b[i] = row * kBK + swz(row, ck) * 16;
-  }
-
-  i32x4 ra[A_CH], rb[B_CH];
-  auto gload = [&](int k0) {
-    const bool in = (k0 + ck * 16) < K;  // K tail: chunks past K read as zero
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) ra[i] = in ? *(const i32x4*)(ga[i] + k0) : i32x4{0, 0, 0, 0};
-#pragma unroll
-    for (int i = 0; i < B_CH; ++i) rb[i] = in ? *(const i32x4*)(gb[i] + k0) : i32x4{0, 0, 0, 0};
+  int a_col[A_CH], b_col[B_CH];  // byte column of this lane's source chunk
+  const int cslot = tid & 7;     // chunk slot within the 128-byte LDS row
+  qmm_static_for<A_CH>([&](auto ic) {
+    constexpr int i = ic;
+    const int row = (i * T + tid) >> 3;
+    a_col[i] = swz(row, cslot) * 16;
+    ga[i] = g.a + (size_t)min(m0 + row, g.M - 1) * K + a_col[i];
+  });
+  qmm_static_for<B_CH>([&](auto ic) {
+    constexpr int i = ic;
+    const int row = (i * T + tid) >> 3;
+    b_col[i] = swz(row, cslot) * 16;
+    gb[i] = g.b + (size_t)min(n0 + row, g.N - 1) * K + b_col[i];
+  });
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto stage_load = [&](int stage, int k0) __attribute__((always_inline)) {
+    char* const wa = sA + stage * BM * kBK + wave * 1024;  // this wave's 1 KB slices: + i * T * 16
+    char* const wb = sB + stage * BN * kBK + wave * 1024;
+    if (k0 + kBK <= K) {  // whole step inside K (uniform): no per-lane conditions
+      qmm_static_for<A_CH>([&](auto ic) {
+        constexpr int i = ic;
+        __builtin_amdgcn_global_load_lds((const void*)(ga[i] + k0), (lds_ptr_t)(wa + i * (T * 16)), 16, 0, 0);
+      });
+      qmm_static_for<B_CH>([&](auto ic) {
+        constexpr int i = ic;
+        __builtin_amdgcn_global_load_lds((const void*)(gb[i] + k0), (lds_ptr_t)(wb + i * (T * 16)), 16, 0, 0);
+      });
+    } else {  // last, partial step: chunks past K are zero-filled
+      qmm_static_for<A_CH>([&](auto ic) {
+        constexpr int i = ic;
+        char* const dst = wa + i * (T * 16);
+        if (k0 + a_col[i] < K) __builtin_amdgcn_global_load_lds((const void*)(ga[i] + k0), (lds_ptr_t)dst, 16, 0, 0);
+        else *(i32x4*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+      });
+      qmm_static_for<B_CH>([&](auto ic) {
+        constexpr int i = ic;
+        char* const dst = wb + i * (T * 16);
+        if (k0 + b_col[i] < K) __builtin_amdgcn_global_load_lds((const void*)(gb[i] + k0), (lds_ptr_t)dst, 16, 0, 0);
+        else *(i32x4*)(dst + lane * 16) = i32x4{0, 0, 0, 0};
+      });
+    }
   };
-  auto sstore = [&](int stage) {
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) *(i32x4*)(sA + stage * BM * kBK + lds_a[i]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < B_CH; ++i) *(i32x4*)(sB + stage * BN * kBK + lds_b[i]) = rb[i];
+  // All of this wave's copies have landed in LDS (they count as vector-memory
+  // operations), then the workgroup meets.
+  auto stage_sync = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), leave expcnt/lgkmcnt alone
+    qmm_lds_barrier();
   };
 
   i32x16 acc[MI][NI];
@@ -117,7 +141,7 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
   const int lrow = lane & 31, lchunk = lane >> 5;
-  auto compute = [&](int stage) {
+  auto compute = [&](int stage) __attribute__((always_inline)) {
     const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
     const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
 #pragma unroll
@@ -143,25 +167,20 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   };
 
   const int ksteps = (K + kBK - 1) / kBK;
-  gload(0);
-  sstore(0);
-  __syncthreads();
+  stage_load(0, 0);
+  stage_sync();
   for (int kt = 0; kt < ksteps; ++kt) {
     const int cur = kt & 1;
-#ifndef QMM_DBG
-#define QMM_DBG 0
-#endif
-    if constexpr (!(QMM_DBG & 1)) { if (kt + 1 < ksteps) gload((kt + 1) * kBK); }
-    if constexpr (!(QMM_DBG & 2)) compute(cur);
-    if constexpr (!(QMM_DBG & 4)) { if (kt + 1 < ksteps) sstore(cur ^ 1); }
-    if constexpr (!(QMM_DBG & 8)) __syncthreads();
+    // stage cur^1 was last read in step kt-1, which every wave has left
+    if (kt + 1 < ksteps) stage_load(cur ^ 1, (kt + 1) * kBK);
+    compute(cur);
+    stage_sync();
   }
 
   // Epilogue, staged through LDS so that (a) the code stays small (the
   // accumulators are register-indexed by constants only in the 16*MI*NI
   // ds_write instructions; everything else is a rolled loop) and (b) global
   // stores are row-contiguous vectors instead of one element per lane.
-  if constexpr (QMM_DBG & 16) { if (acc[0][0][0] != 12345) return; }
   constexpr int kEpStride = TN + 8;  // ints per staged row: +8 keeps rows 16-byte aligned and
                                      // shifts the second half-wave (4 rows down) by 32 banks
   static_assert(4 * WM * WN * 32 * kEpStride + 4 * 4 * (BM + BN) <= 2 * (BM + BN) * kBK,
