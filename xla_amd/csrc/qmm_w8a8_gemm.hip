@@ -43,7 +43,11 @@ struct GemmArgs {
 
 __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
-template <int BM, int BN, int WM, int WN>
+// EPI selects the epilogue: 0 = general (any dtype chain, zero point, raw
+// accumulator output, partial tiles); 1/2/3 = all-f32 scale chain with bf16 /
+// f16 / f32 output and nothing else, which whole tiles finish with a short
+// branch-free loop (partial tiles of such a launch still take the general code).
+template <int BM, int BN, int WM, int WN, int EPI>
 __global__ void __launch_bounds__(WM * WN * 64)
 qmm_w8a8_gemm_kernel(GemmArgs g) {
   constexpr int T = WM * WN * 64;
@@ -132,6 +136,25 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
     qmm_lds_barrier();
   };
 
+  // Scales of this tile are fetched now so that their latency is hidden by the
+  // main loop: thread t keeps x_scale[m0+t] and w_scale[n0+t] (BM, BN <= T).
+  static_assert(BM <= T && BN <= T, "one scale per thread");
+  const bool has_zp = g.zp != nullptr;
+  const bool want_out = g.out != nullptr, want_acc = g.acc_out != nullptr;
+  float pre_xs = 0.f, pre_xsum = 0.f, pre_ws = 0.f, pre_zp = 0.f;
+  if (want_out) {
+    if (tid < BM) {
+      const int m = min(m0 + tid, g.M - 1);
+      pre_xs = qmm_load(g.x_scale, m, g.x_scale_dt);
+      if (has_zp) pre_xsum = qmm_round_dt((float)g.x_sum[m], g.zpo_dt);
+    }
+    if (tid < BN) {
+      const int n = min(n0 + tid, g.N - 1);
+      pre_ws = qmm_load(g.w_scale, n, g.w_scale_dt);
+      if (has_zp) pre_zp = qmm_load(g.zp, n, g.zp_dt);
+    }
+  }
+
   i32x16 acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -141,29 +164,42 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
   const int lrow = lane & 31, lchunk = lane >> 5;
+  // One K step out of LDS: 4 sub-steps of 32 bytes.  The operand fragments of
+  // sub-step ks+1 are read while the MFMAs of sub-step ks run (two register
+  // sets), so the matrix pipe does not wait for LDS latency between sub-steps.
   auto compute = [&](int stage) __attribute__((always_inline)) {
     const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
     const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
-#pragma unroll
-    for (int ks = 0; ks < kBK / 32; ++ks) {
-      i32x4 af[MI], bf[NI];
+    i32x4 af[2][MI], bf[2][NI];
+    auto read_frags = [&](auto setc, auto ksc) __attribute__((always_inline)) {
+      constexpr int set = setc, ks = ksc;
       const int c = 2 * ks + lchunk;
-#pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        int row = i * 32 + lrow;
-        af[i] = *(const i32x4*)(a_base + row * kBK + swz(wm * TM + row, c) * 16);
-      }
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        int row = j * 32 + lrow;
-        bf[j] = *(const i32x4*)(b_base + row * kBK + swz(wn * TN + row, c) * 16);
-      }
-#pragma unroll
-      for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
+      qmm_static_for<MI>([&](auto ic) {
+        constexpr int i = ic;
+        const int row = i * 32 + lrow;
+        af[set][i] = *(const i32x4*)(a_base + row * kBK + swz(wm * TM + row, c) * 16);
+      });
+      qmm_static_for<NI>([&](auto jc) {
+        constexpr int j = jc;
+        const int row = j * 32 + lrow;
+        bf[set][j] = *(const i32x4*)(b_base + row * kBK + swz(wn * TN + row, c) * 16);
+      });
+    };
+    read_frags(qmm_const<0>{}, qmm_const<0>{});
+    qmm_static_for<kBK / 32>([&](auto ksc) {
+      constexpr int ks = ksc, set = ks & 1;
+      if constexpr (ks + 1 < kBK / 32) read_frags(qmm_const<set ^ 1>{}, qmm_const<ks + 1>{});
+      // keep those reads ahead of this sub-step's MFMAs (the scheduler would
+      // otherwise sink each read next to its first use to save registers)
+      __builtin_amdgcn_sched_barrier(0);
+      qmm_static_for<MI>([&](auto ic) {
+        constexpr int i = ic;
+        qmm_static_for<NI>([&](auto jc) {
+          constexpr int j = jc;
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+        });
+      });
+    });
   };
 
   const int ksteps = (K + kBK - 1) / kBK;
@@ -191,26 +227,56 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   float* s_ws = s_xsum + BM;           // [BN] weight scale
   float* s_zp = s_ws + BN;             // [BN] zero point
   int* s_ep = (int*)(s_zp + BN) + wave * (32 * kEpStride);  // per-wave [32][kEpStride]
-  const bool has_zp = g.zp != nullptr;
-  const bool want_out = g.out != nullptr, want_acc = g.acc_out != nullptr;
-  if (want_out) {
-    for (int t = tid; t < BM; t += T) {
-      const int m = min(m0 + t, g.M - 1);
-      s_xs[t] = qmm_load(g.x_scale, m, g.x_scale_dt);
-      s_xsum[t] = has_zp ? qmm_round_dt((float)g.x_sum[m], g.zpo_dt) : 0.f;
-    }
-    for (int t = tid; t < BN; t += T) {
-      const int n = min(n0 + t, g.N - 1);
-      s_ws[t] = qmm_load(g.w_scale, n, g.w_scale_dt);
-      s_zp[t] = has_zp ? qmm_load(g.zp, n, g.zp_dt) : 0.f;
-    }
-  }
+  if (tid < BM) { s_xs[tid] = pre_xs; s_xsum[tid] = pre_xsum; }
+  if (tid < BN) { s_ws[tid] = pre_ws; s_zp[tid] = pre_zp; }
   __syncthreads();
-  const bool simple = g.cvt_dt == XLA_AMD_DT_F32 && g.mid_dt == XLA_AMD_DT_F32 && !has_zp;
-  const bool n_vec = (g.N % 4) == 0;  // rows of out start 8/16-byte aligned
   constexpr int kLanesPerRow = TN / 4;               // each lane finishes 4 consecutive n
   constexpr int kPasses = 32 * kLanesPerRow / 64;    // passes over a 32-row block
+  constexpr int kRowsPerPass = 64 / kLanesPerRow;
 
+  if constexpr (EPI != 0) {
+    if (m0 + BM <= g.M && n0 + BN <= g.N) {
+      // Whole tile, f32 chain: out = cast((float(acc) * w_scale) * x_scale).  The lane's
+      // 4 columns are the same in every pass, so their scales stay in registers.
+      const int c4 = lane % kLanesPerRow, prow = lane / kLanesPerRow;
+      const f32x4 ws = *(const f32x4*)(s_ws + wn * TN + c4 * 4);
+      const int n = n0 + wn * TN + c4 * 4;
+      qmm_static_for<MI>([&](auto ic) {
+        constexpr int i = ic;
+        qmm_static_for<NI>([&](auto jc) {
+          constexpr int j = jc;
+          qmm_static_for<16>([&](auto vc) {
+            constexpr int v = vc;
+            s_ep[(8 * (v >> 2) + 4 * lchunk + (v & 3)) * kEpStride + j * 32 + lrow] = acc[i][j][v];
+          });
+        });
+        const int rbase = wm * TM + i * 32 + prow;
+#pragma unroll 4
+        for (int p = 0; p < kPasses; ++p) {
+          const int row = p * kRowsPerPass;
+          const i32x4 a = *(const i32x4*)(s_ep + (row + prow) * kEpStride + c4 * 4);
+          const float xs = s_xs[rbase + row];
+          const float v0 = ((float)a[0] * ws[0]) * xs, v1 = ((float)a[1] * ws[1]) * xs;
+          const float v2 = ((float)a[2] * ws[2]) * xs, v3 = ((float)a[3] * ws[3]) * xs;
+          const size_t idx0 = (size_t)(m0 + rbase + row) * g.N + n;
+          if constexpr (EPI == 3) {
+            *(f32x4*)((float*)g.out + idx0) = f32x4{v0, v1, v2, v3};
+          } else if constexpr (EPI == 1) {
+            const uint32_t lo = qmm_f32_to_bf16(v0) | ((uint32_t)qmm_f32_to_bf16(v1) << 16);
+            const uint32_t hi = qmm_f32_to_bf16(v2) | ((uint32_t)qmm_f32_to_bf16(v3) << 16);
+            *(i32x2*)((uint16_t*)g.out + idx0) = i32x2{(int)lo, (int)hi};
+          } else {
+            const uint32_t lo = qmm_f32_to_f16(v0) | ((uint32_t)qmm_f32_to_f16(v1) << 16);
+            const uint32_t hi = qmm_f32_to_f16(v2) | ((uint32_t)qmm_f32_to_f16(v3) << 16);
+            *(i32x2*)((uint16_t*)g.out + idx0) = i32x2{(int)lo, (int)hi};
+          }
+        }
+      });
+      return;
+    }
+  }
+  const bool simple = g.cvt_dt == XLA_AMD_DT_F32 && g.mid_dt == XLA_AMD_DT_F32 && !has_zp;
+  const bool n_vec = (g.N % 4) == 0;  // rows of out start 8/16-byte aligned
   // Finishes one staged 32 x TN block whose first row is global row mb.
   auto finish_block = [&](int mb, int row_off) {
     for (int p = 0; p < kPasses; ++p) {
@@ -274,15 +340,15 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   });
 }
 
-template <int BM, int BN, int WM, int WN>
-int launch_tile(GemmArgs g, hipStream_t stream) {
+template <int BM, int BN, int WM, int WN, int EPI>
+int launch_tile_epi(GemmArgs g, hipStream_t stream) {
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   const int ntiles = g.tiles_m * g.tiles_n;
   const int per = (ntiles + 7) / 8;
   const unsigned grid = (unsigned)(per * 8);
   constexpr size_t lds = 2 * (size_t)(BM + BN) * kBK;
-  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN>;
+  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN, EPI>;
   static thread_local bool attr_set = false;
   if (!attr_set) {
     int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
@@ -292,6 +358,18 @@ int launch_tile(GemmArgs g, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, stream, g);
   return QMM_CHECK_LAUNCH("w8a8_gemm launch");
+}
+
+// The short epilogue applies when the scale chain is all f32, there is no zero
+// point, no raw-accumulator output and rows of out are vector-aligned.
+template <int BM, int BN, int WM, int WN>
+int launch_tile(const GemmArgs& g, hipStream_t stream) {
+  const bool fast = g.out && !g.acc_out && !g.zp && g.cvt_dt == XLA_AMD_DT_F32 &&
+                    g.mid_dt == XLA_AMD_DT_F32 && (g.N % 4) == 0 && (((uintptr_t)g.out) & 15) == 0;
+  if (fast && g.out_dt == XLA_AMD_DT_BF16) return launch_tile_epi<BM, BN, WM, WN, 1>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_F16) return launch_tile_epi<BM, BN, WM, WN, 2>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_F32) return launch_tile_epi<BM, BN, WM, WN, 3>(g, stream);
+  return launch_tile_epi<BM, BN, WM, WN, 0>(g, stream);
 }
 
 }  // namespace
