@@ -272,13 +272,29 @@ qmm_skinny_kernel(SkinnyArgs a) {
 
   // End of quantization block sblk: p = round_x(dot); sacc += scale[s,n] * p;
   // zacc += round_x(xsum) * zp[s,n]; the block accumulators restart.
+  // Per-channel: the only scales a lane ever needs are fetched now, so that
+  // their latency is hidden behind the main loop instead of trailing it.
+  float pre_sc[4] = {0.f, 0.f, 0.f, 0.f}, pre_zp[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (RED == kRedRaw) {
+    qmm_static_for<4>([&](auto vc) {
+      constexpr int v = vc;
+      const int n = min(n_wave + 4 * g + v, N - 1);
+      pre_sc[v] = qmm_load(a.scale, n, a.scale_dt);
+      if constexpr (HASZP) pre_zp[v] = qmm_load(a.zp, n, a.zp_dt);
+    });
+  }
   auto block_epilogue = [&](int sblk) __attribute__((always_inline)) {
     qmm_static_for<4>([&](auto vc) {
       constexpr int v = vc;
       const int n = min(n_wave + 4 * g + v, N - 1);
-      const float sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
-      float zv = 0.f;
-      if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
+      float sc, zv = 0.f;
+      if constexpr (RED == kRedRaw) {
+        sc = pre_sc[v];
+        zv = pre_zp[v];
+      } else {
+        sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
+        if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
+      }
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
         const float xsv = NEEDXS ? xs[mt][v] : 0.f;
