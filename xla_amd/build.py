@@ -15,12 +15,16 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 OBJ_DIR = os.path.join(PKG_DIR, "csrc", "build")
 LIB_PATH = os.path.join(PKG_DIR, "libxla_amd_qmm.so")
 
+# (source, extra flags, object name); the skinny kernels are built once per
+# activation dtype so that the three units compile in parallel
 SOURCES = [
-    "qmm_api.hip",
-    "qmm_generic.hip",
-    "qmm_skinny.hip",
-    "qmm_quant_act.hip",
-    "qmm_w8a8_gemm.hip",
+    ("qmm_api.hip", [], "qmm_api.o"),
+    ("qmm_generic.hip", [], "qmm_generic.o"),
+    ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=0"], "qmm_skinny_f32.o"),
+    ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=1"], "qmm_skinny_bf16.o"),
+    ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=2"], "qmm_skinny_f16.o"),
+    ("qmm_quant_act.hip", [], "qmm_quant_act.o"),
+    ("qmm_w8a8_gemm.hip", [], "qmm_w8a8_gemm.o"),
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -44,13 +48,14 @@ def _run(cmd):
   return out
 
 
-def build(verbose: bool = False, jobs: int = 5) -> str:
+def build(verbose: bool = False, jobs: int = 7) -> str:
   os.makedirs(OBJ_DIR, exist_ok=True)
   objs = []
 
-  def compile_one(src):
-    obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
-    out = _run([HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+  def compile_one(item):
+    src, extra, name = item
+    obj = os.path.join(OBJ_DIR, name)
+    out = _run([HIPCC] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
     if verbose and out.strip():
       print(out)
     return obj

@@ -25,11 +25,27 @@
 // in lane (j + 16*(i/4)), register i%4: channel 4g + v, x row r.
 #include "qmm_common.h"
 
-#ifdef QMM_SK_NONT
-#define QMM_SK_LOAD(p) (*(p))
-#else
-#define QMM_SK_LOAD(p) __builtin_nontemporal_load(p)
+// This file is compiled once per activation dtype (-DQMM_SKINNY_XT=0|1|2, the
+// XLA_AMD_DT_* value) so that the three sets of kernels build in parallel; the
+// bf16 unit also holds the C entry point, which calls into the other two.
+#ifndef QMM_SKINNY_XT
+#error "compile with -DQMM_SKINNY_XT=<XLA_AMD_DT_* value>"
 #endif
+
+struct SkinnyArgs {
+  const void* x;
+  const uint8_t* w;  // K-major packed weight
+  const void* scale;
+  const void* zp;
+  void* out;
+  int M, N, K, C;  // M = rows of this pass (<= 16*MT)
+  int scale_dt, zp_dt, out_dt;
+};
+
+int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
+int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
+int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
+
 namespace {
 
 constexpr int kWaves = 4;
@@ -106,15 +122,6 @@ template <int XT> __device__ __forceinline__ i32x4 ones_frag() {
   return o;
 }
 
-struct SkinnyArgs {
-  const void* x;
-  const uint8_t* w;  // K-major packed weight
-  const void* scale;
-  const void* zp;
-  void* out;
-  int M, N, K, C;  // M = rows of this pass (<= 16*MT)
-  int scale_dt, zp_dt, out_dt;
-};
 
 // Reduction over the k-splits of a workgroup.
 constexpr int kRedNone = 0;    // blockwise, KW == 1: nothing to reduce
@@ -134,10 +141,7 @@ struct SkinnyCfg {
   static constexpr int STAGE = W_TILE + KW * X_TILE;
   static constexpr int NS = 2 * STAGE <= kLdsLimit ? 2 : 1;  // LDS stages
   static constexpr int XP = X_TILE / 1024 / RW;              // 1 KB x loads per wave per step
-#ifndef QMM_SK_P
-#define QMM_SK_P 2
-#endif
-  static constexpr int P = ((32 + 4 * XP) <= 64 && QMM_SK_P == 2) ? 2 : 1;      // steps of loads in flight (register ring)
+  static constexpr int P = (32 + 4 * XP) <= 64 ? 2 : 1;      // steps of loads in flight (register ring)
   static constexpr int LDS_BYTES = NS * STAGE;
   static constexpr bool kFits = STAGE <= kLdsLimit;
   static_assert((X_TILE / 1024) % RW == 0, "x tile must split evenly over the waves of a k-split");
@@ -210,7 +214,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
     if ((gs + 1) * KS <= K) {  // whole step inside K: no per-lane conditions
       qmm_static_for<8>([&](auto ic) {
         constexpr int i = ic;
-        wreg[p][i] = QMM_SK_LOAD((const i32x4*)(wp + w_off[i]));
+        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
       });
       qmm_static_for<XP>([&](auto jc) {
         constexpr int j = jc;
@@ -224,7 +228,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
         constexpr int i = ic;
         // w_left >= 64 here, so 0 <= back <= w_chunk * 16 <= w_off[i]
         const int back = max(w_chunk * 16 + 16 - w_left, 0);
-        wreg[p][i] = QMM_SK_LOAD((const i32x4*)(wp + ((int64_t)w_off[i] - back)));
+        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + ((int64_t)w_off[i] - back)));
       });
       qmm_static_for<XP>([&](auto jc) {
         constexpr int j = jc;
@@ -400,11 +404,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // paths only would force the compiler to wait for *all* outstanding loads
   // wherever it needs one of them.
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
-#ifndef QMM_SK_UNROLL
-#define QMM_SK_UNROLL 2
-#endif
-  constexpr int kUnroll = QMM_SK_UNROLL;  // steps per loop trip: the compiler's wait-count bookkeeping is exact
-                              // inside straight-line code and conservative across the back edge
+  constexpr int kUnroll = 2;  // steps per loop trip: covers both ring slots and both LDS stages
   for (int s0 = 0; s0 < trips; s0 += kUnroll) {
     qmm_static_for<kUnroll>([&](auto hc) {
       const int s = s0 + hc;
@@ -506,10 +506,6 @@ qmm_skinny_kernel(SkinnyArgs a) {
   });
 }
 
-#ifdef QMM_SK_PROBE
-template __global__ void qmm_skinny_kernel<XLA_AMD_DT_BF16, 8, 1, 1, kRedRaw, false>(SkinnyArgs);
-}  // namespace
-#else
 template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
 int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
   using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
@@ -573,6 +569,19 @@ int launch_bits(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream) {
 
 }  // namespace
 
+#if QMM_SKINNY_XT == XLA_AMD_DT_F32
+int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream) {
+  return launch_bits<XLA_AMD_DT_F32>(a, bits, haszp, stream);
+}
+#elif QMM_SKINNY_XT == XLA_AMD_DT_F16
+int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream) {
+  return launch_bits<XLA_AMD_DT_F16>(a, bits, haszp, stream);
+}
+#else
+int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream) {
+  return launch_bits<XLA_AMD_DT_BF16>(a, bits, haszp, stream);
+}
+
 extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packed, const void* scale,
                                               const void* zp, void* out, int64_t M, int64_t N,
                                               int64_t K, int64_t C, int bits, int x_dt, int scale_dt,
@@ -609,11 +618,11 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packe
     a.N = (int)N; a.K = (int)K; a.C = (int)C;
     a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.out_dt = out_dt;
     int rc;
-    if (x_dt == XLA_AMD_DT_BF16) rc = launch_bits<XLA_AMD_DT_BF16>(a, bits, zp != nullptr, (hipStream_t)stream);
-    else if (x_dt == XLA_AMD_DT_F16) rc = launch_bits<XLA_AMD_DT_F16>(a, bits, zp != nullptr, (hipStream_t)stream);
-    else rc = launch_bits<XLA_AMD_DT_F32>(a, bits, zp != nullptr, (hipStream_t)stream);
+    if (x_dt == XLA_AMD_DT_BF16) rc = qmm_skinny_launch_bf16(a, bits, zp != nullptr, (hipStream_t)stream);
+    else if (x_dt == XLA_AMD_DT_F16) rc = qmm_skinny_launch_f16(a, bits, zp != nullptr, (hipStream_t)stream);
+    else rc = qmm_skinny_launch_f32(a, bits, zp != nullptr, (hipStream_t)stream);
     if (rc != XLA_AMD_QMM_OK) return rc;
   }
   return XLA_AMD_QMM_OK;
 }
-#endif  // QMM_SK_PROBE
+#endif  // QMM_SKINNY_XT
