@@ -1,7 +1,7 @@
 // Per-token dynamic int8 quantization of activations (HBM-bound elementwise +
-// row reduction).  One workgroup per row; the row is read twice (the second
-// read hits L2: a row is at most a few tens of KB), so x is streamed from HBM
-// once and x_q written once.
+// row reduction).  One workgroup per row.  Rows of up to 8192 elements stay in
+// registers between the abs-max pass and the quantize pass (x is read exactly
+// once); longer rows are read a second time, which hits L2.
 //
 // The arithmetic is the reference's, op by op, in x's dtype:
 //   max = amax(|x|); scale = RN_x(max / 127); r = RN_x(x / scale); q = int8(rint(r))
@@ -35,7 +35,8 @@ __device__ __forceinline__ int quantize_one(float xv, float scale, int x_dt, int
 
 // VEC = elements per thread per step: 8 (16-byte loads of 2-byte types, two
 // for f32) when K % 8 == 0 and the row starts are 16-byte aligned, else 1.
-template <int XT, int VEC>
+// KEEP: vector steps of the row a thread keeps in registers (0 = read twice).
+template <int XT, int VEC, int KEEP>
 __global__ void __launch_bounds__(kThreads)
 qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* __restrict__ x_scale,
                     int32_t* __restrict__ x_sum, int64_t K, int scale_out_dt, int policy) {
@@ -46,7 +47,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
   constexpr int esz = XT == XLA_AMD_DT_F32 ? 4 : 2;
   const char* xrow = (const char*)x + (size_t)m * K * esz;
 
-  auto load_vec = [&](int64_t k, float* f) {
+  auto load_vec = [&](int64_t k, float* f) __attribute__((always_inline)) {
     if constexpr (VEC == 1) {
       f[0] = qmm_load(xrow, k, XT);
     } else if constexpr (XT == XLA_AMD_DT_F32) {
@@ -72,13 +73,29 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
 
   // pass 1: row abs-max
   float mx = 0.f;
-  for (int64_t k = (int64_t)tid * VEC; k < K; k += (int64_t)kThreads * VEC) {
-    float f[VEC];
-    load_vec(k, f);
+  float held[KEEP > 0 ? KEEP : 1][VEC];
+  if constexpr (KEEP > 0) {
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      float av = fabsf(f[i]);
-      mx = (av > mx || av != av) ? av : mx;  // propagate NaN like torch.amax
+    for (int s = 0; s < KEEP; ++s) {
+      const int64_t k = ((int64_t)s * kThreads + tid) * VEC;
+      if (k < K) {
+        load_vec(k, held[s]);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          float av = fabsf(held[s][i]);
+          mx = (av > mx || av != av) ? av : mx;
+        }
+      }
+    }
+  } else {
+    for (int64_t k = (int64_t)tid * VEC; k < K; k += (int64_t)kThreads * VEC) {
+      float f[VEC];
+      load_vec(k, f);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        float av = fabsf(f[i]);
+        mx = (av > mx || av != av) ? av : mx;  // propagate NaN like torch.amax
+      }
     }
   }
   mx = wave_max(mx);
@@ -91,9 +108,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
 
   // pass 2: quantize
   int lsum = 0;
-  for (int64_t k = (int64_t)tid * VEC; k < K; k += (int64_t)kThreads * VEC) {
-    float f[VEC];
-    load_vec(k, f);
+  auto emit = [&](int64_t k, const float* f) __attribute__((always_inline)) {
     int q[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
@@ -111,6 +126,19 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
       }
       i32x2 v = {(int)lo, (int)hi};
       *(i32x2*)(xq + (size_t)m * K + k) = v;
+    }
+  };
+  if constexpr (KEEP > 0) {
+#pragma unroll
+    for (int s = 0; s < KEEP; ++s) {
+      const int64_t k = ((int64_t)s * kThreads + tid) * VEC;
+      if (k < K) emit(k, held[s]);
+    }
+  } else {
+    for (int64_t k = (int64_t)tid * VEC; k < K; k += (int64_t)kThreads * VEC) {
+      float f[VEC];
+      load_vec(k, f);
+      emit(k, f);
     }
   }
   if (tid == 0) qmm_store(x_scale, m, scale, scale_out_dt);
@@ -130,12 +158,15 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
 template <int XT>
 int launch(const void* x, int8_t* xq, void* x_scale, int32_t* x_sum, int64_t M, int64_t K,
            int scale_out_dt, int policy, bool vec, hipStream_t stream) {
-  if (vec)
-    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8>), dim3((unsigned)M), dim3(kThreads), 0, stream, x,
-                       xq, x_scale, x_sum, K, scale_out_dt, policy);
+  const dim3 grid((unsigned)M), block(kThreads);
+  if (!vec)
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 1, 0>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
+  else if (K <= 2 * kThreads * 8)
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 2>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
+  else if (K <= 4 * kThreads * 8)
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 4>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
   else
-    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 1>), dim3((unsigned)M), dim3(kThreads), 0, stream, x,
-                       xq, x_scale, x_sum, K, scale_out_dt, policy);
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 0>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
   return QMM_CHECK_LAUNCH("quantize_per_token launch");
 }
 
