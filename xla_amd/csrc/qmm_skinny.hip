@@ -159,7 +159,9 @@ qmm_skinny_kernel(SkinnyArgs a) {
   constexpr int XQ = kMfma ? 4 : 8;                       // 16-byte x chunks per lane per sub-step
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  // wave-uniform values live in scalar registers: branches on them are scalar branches
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rw = wave % RW, kw = wave / RW;
   const int r = lane & 15, g = lane >> 4;
   const int K = a.K, N = a.N, M = a.M, C = a.C;
@@ -325,102 +327,128 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const char* xb = smem + stage * STAGE + W_TILE + kw * X_TILE;
     const int k_step = (s * KW + kw) * KS;
     if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
-    qmm_static_for<SUB>([&](auto tc) {
+    // fragments of sub-step t: this lane's 32 weight bytes and, per tile of 16
+    // x rows, its XQ 16-byte chunks of x
+    auto read_frags = [&](auto tc, i32x4& wq0, i32x4& wq1, i32x4 (&xq)[MT][XQ]) __attribute__((always_inline)) {
+      constexpr int t = tc;
+      if constexpr (BITS == 8) {
+        wq0 = *(const i32x4*)(wb + (((8 * t + 2 * g) ^ r) * 16));
+        wq1 = *(const i32x4*)(wb + (((8 * t + 2 * g + 1) ^ r) * 16));
+      } else {
+        wq0 = *(const i32x4*)(wb + (((4 * t + g) ^ r) * 16));
+        wq1 = wq0;
+      }
+      qmm_static_for<MT>([&](auto mc) {
+        constexpr int mt = mc;
+        qmm_static_for<XQ>([&](auto qc) {
+          constexpr int q = qc;
+          xq[mt][q] = *(const i32x4*)(xb + (16 * mt + r) * XROW + (((XQ * 4 * t + XQ * g + q) ^ r) * 16));
+        });
+      });
+    };
+    auto math = [&](auto tc, const i32x4& wq0, const i32x4& wq1, const i32x4 (&xq)[MT][XQ]) __attribute__((always_inline)) {
       constexpr int t = tc;
       const int k_sub = k_step + t * 128;
-      if (kFull || k_sub < K) {
-        i32x4 wq0, wq1;
-        if constexpr (BITS == 8) {
-          wq0 = *(const i32x4*)(wb + (((8 * t + 2 * g) ^ r) * 16));
-          wq1 = *(const i32x4*)(wb + (((8 * t + 2 * g + 1) ^ r) * 16));
-        } else {
-          wq0 = *(const i32x4*)(wb + (((4 * t + g) ^ r) * 16));
-          wq1 = wq0;
-        }
-        i32x4 xq[MT][XQ];
-        qmm_static_for<MT>([&](auto mc) {
-          constexpr int mt = mc;
-          qmm_static_for<XQ>([&](auto qc) {
-            constexpr int q = qc;
-            xq[mt][q] = *(const i32x4*)(xb + (16 * mt + r) * XROW + (((XQ * 4 * t + XQ * g + q) ^ r) * 16));
+      if constexpr (kMfma) {
+        qmm_static_for<4>([&](auto jc) {
+          constexpr int j = jc;
+          i32x4 af;
+          if constexpr (BITS == 8) {
+            const i32x4 src = (j >> 1) ? wq1 : wq0;
+            af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
+          } else {
+            af = cvt_w4<XT>((uint32_t)wq0[j]);
+          }
+          qmm_static_for<MT>([&](auto mc) {
+            constexpr int mt = mc;
+            if constexpr (j & 1) accb[mt] = mfma16<XT>(af, xq[mt][j], accb[mt]);
+            else acc[mt] = mfma16<XT>(af, xq[mt][j], acc[mt]);
+            if constexpr (NEEDXS) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt][j], xs[mt]);
           });
         });
-        if constexpr (kMfma) {
-          qmm_static_for<4>([&](auto jc) {
-            constexpr int j = jc;
-            i32x4 af;
-            if constexpr (BITS == 8) {
-              const i32x4 src = (j >> 1) ? wq1 : wq0;
-              af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
-            } else {
-              af = cvt_w4<XT>((uint32_t)wq0[j]);
-            }
-            qmm_static_for<MT>([&](auto mc) {
-              constexpr int mt = mc;
-              if constexpr (j & 1) accb[mt] = mfma16<XT>(af, xq[mt][j], accb[mt]);
-              else acc[mt] = mfma16<XT>(af, xq[mt][j], acc[mt]);
-              if constexpr (NEEDXS) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt][j], xs[mt]);
-            });
-          });
-        } else {
-          // f32 x: 16x16x4 f32 MFMA, one column per lane per instruction.
-          qmm_static_for<32>([&](auto kc) {
-            constexpr int kk = kc;  // 0..31 within the lane's columns
-            float wf;
-            if constexpr (BITS == 8) {
-              const i32x4 src = (kk >> 4) ? wq1 : wq0;
-              const uint32_t dw = (uint32_t)src[(kk >> 2) & 3];
-              wf = (float)(int8_t)(dw >> (8 * (kk & 3)));
-            } else {
-              // column kk = 8*word + P[nibble]: nibble = (c&1)*4 + (c>>1), c = kk % 8
-              const uint32_t dw = (uint32_t)wq0[kk >> 3];
-              constexpr int c = kk & 7, nib = (c & 1) * 4 + (c >> 1);
-              wf = (float)(int)((dw >> (4 * nib)) & 15u) - 8.0f;
-            }
-            qmm_static_for<MT>([&](auto mc) {
-              constexpr int mt = mc;
-              constexpr int xq_i = kk >> 2, xe_i = kk & 3;
-              const f32x4 xv4 = __builtin_bit_cast(f32x4, xq[mt][xq_i]);
-              const float xv = xv4[xe_i];
-              if constexpr (kk & 1) accb[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv, accb[mt], 0, 0, 0);
-              else acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv, acc[mt], 0, 0, 0);
-              if constexpr (NEEDXS) xs[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, xv, xs[mt], 0, 0, 0);
-            });
-          });
-        }
-        if constexpr (RED != kRedRaw) {
-          if (--block_left == 0) {
-            block_epilogue(k_sub / C);
-            block_left = sub_per_block;
+      } else {
+        // f32 x: 16x16x4 f32 MFMA, one column per lane per instruction.
+        qmm_static_for<32>([&](auto kc) {
+          constexpr int kk = kc;  // 0..31 within the lane's columns
+          float wf;
+          if constexpr (BITS == 8) {
+            const i32x4 src = (kk >> 4) ? wq1 : wq0;
+            const uint32_t dw = (uint32_t)src[(kk >> 2) & 3];
+            wf = (float)(int8_t)(dw >> (8 * (kk & 3)));
+          } else {
+            // column kk = 8*word + P[nibble]: nibble = (c&1)*4 + (c>>1), c = kk % 8
+            const uint32_t dw = (uint32_t)wq0[kk >> 3];
+            constexpr int c = kk & 7, nib = (c & 1) * 4 + (c >> 1);
+            wf = (float)(int)((dw >> (4 * nib)) & 15u) - 8.0f;
           }
+          qmm_static_for<MT>([&](auto mc) {
+            constexpr int mt = mc;
+            constexpr int xq_i = kk >> 2, xe_i = kk & 3;
+            const f32x4 xv4 = __builtin_bit_cast(f32x4, xq[mt][xq_i]);
+            const float xv = xv4[xe_i];
+            if constexpr (kk & 1) accb[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv, accb[mt], 0, 0, 0);
+            else acc[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wf, xv, acc[mt], 0, 0, 0);
+            if constexpr (NEEDXS) xs[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(1.0f, xv, xs[mt], 0, 0, 0);
+          });
+        });
+      }
+      if constexpr (RED != kRedRaw) {
+        if (--block_left == 0) {
+          block_epilogue(k_sub / C);
+          block_left = sub_per_block;
         }
       }
-    });
+    };
+    // (two x tiles with per-block scale accumulators leave no registers for the second fragment set)
+    constexpr bool kPipe = kFull && kMfma && !(MT == 2 && RED == kRedScaled);
+    if constexpr (kPipe) {
+      // Whole step: the LDS reads of sub-step t+1 are issued before the math of
+      // sub-step t (a lone wave per SIMD has nobody else to hide LDS latency).
+      i32x4 wq0[2], wq1[2], xq[2][MT][XQ];
+      read_frags(qmm_const<0>{}, wq0[0], wq1[0], xq[0]);
+      qmm_static_for<SUB>([&](auto tc) {
+        constexpr int t = tc;
+        constexpr int cur = t & 1, nxt = cur ^ 1;
+        if constexpr (t + 1 < SUB) read_frags(qmm_const<t + 1>{}, wq0[nxt], wq1[nxt], xq[nxt]);
+        __builtin_amdgcn_sched_barrier(0);
+        math(tc, wq0[cur], wq1[cur], xq[cur]);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    } else {
+      qmm_static_for<SUB>([&](auto tc) {
+        constexpr int t = tc;
+        if (kFull || k_step + t * 128 < K) {
+          i32x4 wq0, wq1, xq[MT][XQ];
+          read_frags(tc, wq0, wq1, xq);
+          math(tc, wq0, wq1, xq);
+        }
+      });
+    }
   };
 
   // ---- main loop: registers hold loads of P steps ahead, LDS holds NS stages -----------
   // Loads are issued unconditionally, also for steps past the end (those take
-  // the clamped path and are never consumed): a load that is issued on some
-  // paths only would force the compiler to wait for *all* outstanding loads
-  // wherever it needs one of them.
+  // the clamped path): a load that is issued on some paths only would force the
+  // compiler to wait for *all* outstanding loads wherever it needs one of them.
+  // For the same reason every trip also stores the ring slot to LDS and meets
+  // the barrier unconditionally, including the half trip past the end when the
+  // number of trips is odd; what such a trip puts into LDS is never read.
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
-  constexpr int kUnroll = 2;  // steps per loop trip: covers both ring slots and both LDS stages
+  constexpr int kUnroll = (P % 2 == 0) ? (P > 2 ? P : 2) : 2 * P;  // a multiple of the ring depth and of the LDS stages
   for (int s0 = 0; s0 < trips; s0 += kUnroll) {
     qmm_static_for<kUnroll>([&](auto hc) {
       const int s = s0 + hc;
-      if (s < trips) {
-        constexpr int p = hc % P;
-        const int stage = NS == 2 ? (int)(hc % 2) : 0;
-        if constexpr (NS == 1) {
-          if (s > 0) qmm_lds_barrier();  // the single stage is free again
-        }
-        if (s < my_steps) store_lds(qmm_const<p>{}, stage);
-        load_regs(qmm_const<p>{}, s + P);
-        qmm_lds_barrier();
-        if (s < my_steps) {
-          if (((s * KW + kw) + 1) * KS <= K) compute(qmm_const<1>{}, stage, s);
-          else compute(qmm_const<0>{}, stage, s);
-        }
+      constexpr int p = hc % P;
+      const int stage = NS == 2 ? (int)(hc % 2) : 0;
+      if constexpr (NS == 1) {
+        if (s > 0) qmm_lds_barrier();  // the single stage is free again
+      }
+      store_lds(qmm_const<p>{}, stage);
+      load_regs(qmm_const<p>{}, s + P);
+      qmm_lds_barrier();
+      if (s < my_steps) {
+        if (((s * KW + kw) + 1) * KS <= K) compute(qmm_const<1>{}, stage, s);
+        else compute(qmm_const<0>{}, stage, s);
       }
     });
   }

@@ -60,7 +60,8 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   char* sA = smem;                      // [2][BM][128]
   char* sB = smem + 2 * BM * kBK;       // [2][BN][128]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases in scalar registers
   const int wm = wave / WN, wn = wave % WN;
 
   // Workgroup -> tile.  Consecutive workgroup ids go to different XCDs (8 of
@@ -167,7 +168,7 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   // One K step out of LDS: 4 sub-steps of 32 bytes.  The operand fragments of
   // sub-step ks+1 are read while the MFMAs of sub-step ks run (two register
   // sets), so the matrix pipe does not wait for LDS latency between sub-steps.
-  auto compute = [&](int stage) __attribute__((always_inline)) {
+  auto compute = [&](int stage, auto&& after_first_reads) __attribute__((always_inline)) {
     const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
     const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
     i32x4 af[2][MI], bf[2][NI];
@@ -186,6 +187,8 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
       });
     };
     read_frags(qmm_const<0>{}, qmm_const<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    after_first_reads();  // the next stage's copies are issued while those reads are in flight
     qmm_static_for<kBK / 32>([&](auto ksc) {
       constexpr int ks = ksc, set = ks & 1;
       if constexpr (ks + 1 < kBK / 32) read_frags(qmm_const<set ^ 1>{}, qmm_const<ks + 1>{});
@@ -208,8 +211,9 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   for (int kt = 0; kt < ksteps; ++kt) {
     const int cur = kt & 1;
     // stage cur^1 was last read in step kt-1, which every wave has left
-    if (kt + 1 < ksteps) stage_load(cur ^ 1, (kt + 1) * kBK);
-    compute(cur);
+    compute(cur, [&]() __attribute__((always_inline)) {
+      if (kt + 1 < ksteps) stage_load(cur ^ 1, (kt + 1) * kBK);
+    });
     stage_sync();
   }
 
