@@ -1,21 +1,30 @@
 // Weight-streaming GEMV / skinny GEMM for weight-only quantized linear layers
 // on gfx950.  HBM-bound: every weight byte is read from memory exactly once.
 //
-// Memory access.  Global loads are issued so that one wave instruction reads
-// long contiguous runs (2 weight rows x 512 B, or 1 KB of one x row): that is
-// what the memory system streams fastest.  The matrix cores want the opposite
-// arrangement (lane = row, 8 consecutive k per lane), so tiles take one trip
-// through LDS: written as they were loaded, read back in MFMA operand order.
+// Memory access.  Weight loads are issued so that one wave instruction reads
+// long contiguous runs (2 weight rows x 512 B): that is what the memory system
+// streams fastest.  The matrix cores want the opposite arrangement (lane = row,
+// 8 consecutive k per lane), so a wave's weights take one trip through its own
+// LDS tile: written as they were loaded, read back in MFMA operand order.
 // 16-byte chunks are XOR-swizzled with the row number so that both directions
-// are free of bank conflicts.
+// are free of bank conflicts.  The activations are copied global -> LDS without
+// passing registers, a chunk of up to 128 KB of x columns at a time (all of x
+// for 16 rows x 4096 bf16 columns), and stay there while the weights stream by.
 //
 // Work split.  A workgroup has 4 waves arranged as RW row groups x KW k-splits
 // (RW * KW == 4).  It owns 16*RW consecutive output channels.  K is walked in
-// steps of KS columns per k-split (512 B of weight row: 512 columns of int8,
-// 1024 of int4); wave (rw, kw) handles steps kw, kw + KW, ...  The x tile of a
-// step ([16*MT rows] x KS columns) is shared by the RW waves of a k-split.
-// Large N uses RW = 4 (no cross-wave reduction at all); small N trades row
-// groups for k-splits so that the grid still covers the chip.
+// steps of KS columns (512 B of weight row: 512 columns of int8, 1024 of int4);
+// wave (rw, kw) handles steps kw, kw + KW, ...  Large N uses RW = 4 (no
+// cross-wave reduction at all); small N trades row groups for k-splits so that
+// the grid still covers the chip.
+//
+// Synchronisation.  The workgroup meets only when the resident x columns are
+// replaced.  In between nothing is shared but read-only x, so every wave runs
+// at its own pace: wait for its weight loads (a ring of two steps in flight,
+// re-issued piecewise between the multiplies), transpose, multiply.  The waves
+// of a compute unit drift apart, and the memory waits of one overlap the LDS
+// traffic and arithmetic of the others; a barrier per step would instead make
+// each step as slow as its slowest wave.
 //
 // MFMA mapping.  Lane l is (r = l%16, g = l/16).  For a sub-step of 128
 // columns the lane supplies, for weight row r and for x row r of each 16-row
@@ -136,15 +145,15 @@ struct SkinnyCfg {
   static constexpr int SUB = KS / 128;                       // 128-column sub-steps per step
   static constexpr int XROW = KS * XB;                       // bytes of one x row per step
   static constexpr int XROWS = 16 * MT;
-  static constexpr int W_TILE = kWaves * 16 * kWSeg;         // 32 KB: every wave's 16 rows x 512 B
-  static constexpr int X_TILE = XROWS * XROW;                // per k-split
-  static constexpr int STAGE = W_TILE + KW * X_TILE;
-  static constexpr int NS = 2 * STAGE <= kLdsLimit ? 2 : 1;  // LDS stages
-  static constexpr int XP = X_TILE / 1024 / RW;              // 1 KB x loads per wave per step
-  static constexpr int P = (32 + 4 * XP) <= 64 ? 2 : 1;      // steps of loads in flight (register ring)
-  static constexpr int LDS_BYTES = NS * STAGE;
-  static constexpr bool kFits = STAGE <= kLdsLimit;
-  static_assert((X_TILE / 1024) % RW == 0, "x tile must split evenly over the waves of a k-split");
+  static constexpr int W_TILE = kWaves * 16 * kWSeg;         // 32 KB: every wave's private 16 rows x 512 B
+  static constexpr int X_TILE = XROWS * XROW;                // the x columns of one step, all rows
+  static constexpr int CH = (kLdsLimit - W_TILE) / X_TILE;   // steps whose x columns are resident in LDS together
+  static constexpr int XPW = X_TILE / 1024 / kWaves;         // 1 KB pieces of an x tile copied by each wave
+  static constexpr int P = 2;                                // steps of weight loads in flight (register ring)
+  static constexpr int CHG = CH / (2 * KW) * (2 * KW);       // ... rounded so that a chunk holds an even number of steps of every wave
+  static constexpr bool kFits = CHG >= 2 * KW;
+  static constexpr int lds_bytes(int steps) { return W_TILE + (steps < CHG ? steps : CHG) * X_TILE; }
+  static_assert((X_TILE / 1024) % kWaves == 0, "x tile must split evenly over the waves");
 };
 
 template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
@@ -152,8 +161,7 @@ __global__ void __launch_bounds__(kWaves * 64)
 qmm_skinny_kernel(SkinnyArgs a) {
   using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
   constexpr int RW = Cfg::RW, XB = Cfg::XB, KS = Cfg::KS, SUB = Cfg::SUB, XROW = Cfg::XROW;
-  constexpr int W_TILE = Cfg::W_TILE, X_TILE = Cfg::X_TILE, STAGE = Cfg::STAGE, NS = Cfg::NS;
-  constexpr int XP = Cfg::XP, P = Cfg::P;
+  constexpr int W_TILE = Cfg::W_TILE, X_TILE = Cfg::X_TILE, XPW = Cfg::XPW, P = Cfg::P;
   constexpr bool kMfma = XT != XLA_AMD_DT_F32;
   constexpr bool NEEDXS = HASZP || (BITS == 4 && kMfma);  // x sums: zero point, int4 affine map
   constexpr int XQ = kMfma ? 4 : 8;                       // 16-byte x chunks per lane per sub-step
@@ -186,72 +194,89 @@ qmm_skinny_kernel(SkinnyArgs a) {
     w_off[i] = (uint32_t)(n - n_wg) * (uint32_t)row_bytes + w_chunk * 16;
     w_dst[i] = wave * (16 * kWSeg) + row * kWSeg + ((w_chunk ^ row) * 16);
   });
-  // x: piece j of this wave is 1 KB of one row of the k-split's tile
-  uint32_t x_off[XP];
-  int x_dst[XP];
-  qmm_static_for<XP>([&](auto jc) {
+  // x: copied global -> LDS without passing registers (global_load_lds_dwordx4:
+  // lane l of an instruction lands at base + 16 l).  Piece j of this wave is
+  // 1 KB of one row of a step's tile; the XOR swizzle of the tile is applied on
+  // the source side: LDS slot c' of a row receives global chunk c' ^ (row % 16).
+  uint32_t x_off[XPW];  // per lane: byte offset of its source chunk from the step's first column of row 0
+  int x_col[XPW];       // per lane: byte column of that chunk within the step
+  int x_lds[XPW];       // uniform: LDS offset of the piece within a tile
+  qmm_static_for<XPW>([&](auto jc) {
     constexpr int j = jc;
     constexpr int kPiecesPerRow = XROW / 1024;
-    const int q = rw * XP + j;
-    const int row = q / kPiecesPerRow, chunk = (q % kPiecesPerRow) * 64 + lane;
+    const int q = wave * XPW + j;
+    const int row = q / kPiecesPerRow, piece = q % kPiecesPerRow;
     const int m = min(row, M - 1);
-    x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + chunk * 16;
-    x_dst[j] = W_TILE + kw * X_TILE + row * XROW + ((chunk ^ (row & 15)) * 16);
+    x_col[j] = (piece * 64 + (lane ^ (row & 15))) * 16;
+    x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + x_col[j];
+    x_lds[j] = W_TILE + row * XROW + piece * 1024;
   });
 
   const int steps_total = (K + KS - 1) / KS;
   const int my_steps = steps_total > kw ? (steps_total - kw + KW - 1) / KW : 0;
-  // every wave of the workgroup runs the same number of loop trips (barriers)
-  const int trips = (steps_total + KW - 1) / KW;
 
   i32x4 wreg[P][8];
-  i32x4 xreg[P][XP];
-  auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {  // s: this wave's s-th step
-    constexpr int p = pc;
+  // Weight loads number lo..hi-1 of a step's 8 into ring slot p.
+  auto load_range = [&](auto pc, int s, auto loc, auto hic) __attribute__((always_inline)) {  // s: this wave's s-th step
+    constexpr int p = pc, lo = loc, hi = hic;
     // global step; steps past the end (issued only to keep the number of
     // outstanding loads the same on every path) re-read the last real step
     const int gs = min(s * KW + kw, steps_total - 1);
     const uint8_t* const wp = w_base + (size_t)gs * kWSeg;
-    const char* const xp = x_base + (size_t)gs * XROW;
     if ((gs + 1) * KS <= K) {  // whole step inside K: no per-lane conditions
       qmm_static_for<8>([&](auto ic) {
         constexpr int i = ic;
-        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
-      });
-      qmm_static_for<XP>([&](auto jc) {
-        constexpr int j = jc;
-        xreg[p][j] = *(const i32x4*)(xp + x_off[j]);
+        if constexpr (i >= lo && i < hi) wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
       });
     } else {
       // last, partial step: columns past K re-read the last valid 16 bytes of the
       // row (their sub-steps are never computed)
-      const int w_left = row_bytes - gs * kWSeg, x_left = K * XB - gs * XROW;
+      const int w_left = row_bytes - gs * kWSeg;
       qmm_static_for<8>([&](auto ic) {
         constexpr int i = ic;
-        // w_left >= 64 here, so 0 <= back <= w_chunk * 16 <= w_off[i]
-        const int back = max(w_chunk * 16 + 16 - w_left, 0);
-        wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + ((int64_t)w_off[i] - back)));
-      });
-      qmm_static_for<XP>([&](auto jc) {
-        constexpr int j = jc;
-        constexpr int kPiecesPerRow = XROW / 1024;
-        const int col = (((rw * XP + j) % kPiecesPerRow) * 64 + lane) * 16;
-        // x_left >= 256 here, so 0 <= back <= col <= x_off[j]
-        const int back = max(col + 16 - x_left, 0);
-        xreg[p][j] = *(const i32x4*)(xp + ((int64_t)x_off[j] - back));
+        if constexpr (i >= lo && i < hi) {
+          // w_left >= 64 here, so 0 <= back <= w_chunk * 16 <= w_off[i]
+          const int back = max(w_chunk * 16 + 16 - w_left, 0);
+          wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + ((int64_t)w_off[i] - back)));
+        }
       });
     }
   };
-  auto store_lds = [&](auto pc, int stage) __attribute__((always_inline)) {
+  auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {
+    load_range(pc, s, qmm_const<0>{}, qmm_const<8>{});
+  };
+  // The x columns of global steps c0 .. c0+nst-1 into the LDS tiles 0 .. nst-1.
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto x_chunk_load = [&](int c0, int nst) __attribute__((always_inline)) {
+    for (int t = 0; t < nst; ++t) {
+      const int gs = c0 + t;
+      const char* const xp = x_base + (size_t)gs * XROW;
+      char* const tile = smem + t * X_TILE;
+      if ((gs + 1) * KS <= K) {
+        qmm_static_for<XPW>([&](auto jc) {
+          constexpr int j = jc;
+          __builtin_amdgcn_global_load_lds((const void*)(xp + x_off[j]), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
+        });
+      } else {
+        // last, partial step: chunks past K re-read the last valid 16 bytes of the row
+        const int x_left = K * XB - gs * XROW;
+        qmm_static_for<XPW>([&](auto jc) {
+          constexpr int j = jc;
+          // x_left >= 256 here, so 0 <= back <= x_col[j] <= x_off[j]
+          const int back = max(x_col[j] + 16 - x_left, 0);
+          __builtin_amdgcn_global_load_lds((const void*)(xp + ((int64_t)x_off[j] - back)), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
+        });
+      }
+    }
+  };
+  // ring slot p -> this wave's private weight tile (swizzled).  Nobody else
+  // touches that tile and a wave's LDS operations execute in order, so neither
+  // a second stage nor a barrier is needed around it.
+  auto store_w = [&](auto pc) __attribute__((always_inline)) {
     constexpr int p = pc;
-    char* base = smem + stage * STAGE;
     qmm_static_for<8>([&](auto ic) {
       constexpr int i = ic;
-      *(i32x4*)(base + w_dst[i]) = wreg[p][i];
-    });
-    qmm_static_for<XP>([&](auto jc) {
-      constexpr int j = jc;
-      *(i32x4*)(base + x_dst[j]) = xreg[p][j];
+      *(i32x4*)(smem + w_dst[i]) = wreg[p][i];
     });
   };
 
@@ -321,10 +346,13 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // Sub-steps (128 columns) left in the current quantization block; uniform.
   const int sub_per_block = C / 128;
   int block_left = sub_per_block;
-  auto compute = [&](auto fullc, int stage, int s) __attribute__((always_inline)) {
-    constexpr bool kFull = fullc != 0;  // the whole step lies inside K
-    const char* wb = smem + stage * STAGE + wave * (16 * kWSeg) + r * kWSeg;
-    const char* xb = smem + stage * STAGE + W_TILE + kw * X_TILE;
+  // issue(t) is called once per sub-step t = 0..SUB-1, before that sub-step's math:
+  // the caller spreads the next loads over the step with it.  Sub-steps at or
+  // beyond K are skipped (a uniform branch around arithmetic only: the loads stay
+  // in straight-line code, so the compiler's wait counts for the ring stay exact).
+  auto compute = [&](int tile, int s, auto&& issue) __attribute__((always_inline)) {
+    const char* wb = smem + wave * (16 * kWSeg) + r * kWSeg;
+    const char* xb = smem + W_TILE + tile * X_TILE;
     const int k_step = (s * KW + kw) * KS;
     if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
     // fragments of sub-step t: this lane's 32 weight bytes and, per tile of 16
@@ -400,24 +428,26 @@ qmm_skinny_kernel(SkinnyArgs a) {
       }
     };
     // (two x tiles with per-block scale accumulators leave no registers for the second fragment set)
-    constexpr bool kPipe = kFull && kMfma && !(MT == 2 && RED == kRedScaled);
+    constexpr bool kPipe = kMfma && !(MT == 2 && RED == kRedScaled);
     if constexpr (kPipe) {
-      // Whole step: the LDS reads of sub-step t+1 are issued before the math of
-      // sub-step t (a lone wave per SIMD has nobody else to hide LDS latency).
+      // The LDS reads of sub-step t+1 are issued before the math of sub-step t
+      // (a lone wave per SIMD has nobody else to hide LDS latency).
       i32x4 wq0[2], wq1[2], xq[2][MT][XQ];
       read_frags(qmm_const<0>{}, wq0[0], wq1[0], xq[0]);
       qmm_static_for<SUB>([&](auto tc) {
         constexpr int t = tc;
         constexpr int cur = t & 1, nxt = cur ^ 1;
         if constexpr (t + 1 < SUB) read_frags(qmm_const<t + 1>{}, wq0[nxt], wq1[nxt], xq[nxt]);
+        issue(tc);
         __builtin_amdgcn_sched_barrier(0);
-        math(tc, wq0[cur], wq1[cur], xq[cur]);
+        if (k_step + t * 128 < K) math(tc, wq0[cur], wq1[cur], xq[cur]);
         __builtin_amdgcn_sched_barrier(0);
       });
     } else {
+      qmm_static_for<SUB>([&](auto tc) { issue(tc); });
       qmm_static_for<SUB>([&](auto tc) {
         constexpr int t = tc;
-        if (kFull || k_step + t * 128 < K) {
+        if (k_step + t * 128 < K) {
           i32x4 wq0, wq1, xq[MT][XQ];
           read_frags(tc, wq0, wq1, xq);
           math(tc, wq0, wq1, xq);
@@ -426,31 +456,49 @@ qmm_skinny_kernel(SkinnyArgs a) {
     }
   };
 
-  // ---- main loop: registers hold loads of P steps ahead, LDS holds NS stages -----------
-  // Loads are issued unconditionally, also for steps past the end (those take
-  // the clamped path): a load that is issued on some paths only would force the
-  // compiler to wait for *all* outstanding loads wherever it needs one of them.
-  // For the same reason every trip also stores the ring slot to LDS and meets
-  // the barrier unconditionally, including the half trip past the end when the
-  // number of trips is odd; what such a trip puts into LDS is never read.
+  // ---- main loop ---------------------------------------------------------------------
+  // The x columns of a chunk of up to CHG steps are resident in LDS; the workgroup
+  // meets only when they are replaced, and between those points every wave runs
+  // its steps at its own pace (wait for its weights, transpose them through its
+  // private tile, multiply), so that the waves of a compute unit drift apart and
+  // their memory waits, LDS traffic and arithmetic overlap.
+  // Every wave runs the chunk loop the same number of times, whether it has
+  // steps in a chunk or not: the barriers always match.  A chunk holds an even
+  // number of steps of every wave, so each chunk starts on ring slot 0.
+  //
+  // Weight loads are issued unconditionally, also for steps past the end (those
+  // take the clamped path): a load that is issued on some paths only would force
+  // the compiler to wait for *all* outstanding loads wherever it needs one of
+  // them.  For the same reason every half trip stores its ring slot to LDS,
+  // including the one past the end when the number of steps is odd.
+  constexpr int CHG = Cfg::CHG;
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
-  constexpr int kUnroll = (P % 2 == 0) ? (P > 2 ? P : 2) : 2 * P;  // a multiple of the ring depth and of the LDS stages
-  for (int s0 = 0; s0 < trips; s0 += kUnroll) {
-    qmm_static_for<kUnroll>([&](auto hc) {
-      const int s = s0 + hc;
-      constexpr int p = hc % P;
-      const int stage = NS == 2 ? (int)(hc % 2) : 0;
-      if constexpr (NS == 1) {
-        if (s > 0) qmm_lds_barrier();  // the single stage is free again
-      }
-      store_lds(qmm_const<p>{}, stage);
-      load_regs(qmm_const<p>{}, s + P);
-      qmm_lds_barrier();
-      if (s < my_steps) {
-        if (((s * KW + kw) + 1) * KS <= K) compute(qmm_const<1>{}, stage, s);
-        else compute(qmm_const<0>{}, stage, s);
-      }
-    });
+  int s0 = 0;  // this wave's next step
+  for (int c0 = 0; c0 < steps_total; c0 += CHG) {
+    const int nst = min(CHG, steps_total - c0);
+    if (c0 > 0) qmm_lds_barrier();       // every wave has finished reading the old columns
+    x_chunk_load(c0, nst);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+    qmm_lds_barrier();
+    const int s_end = min(my_steps, (c0 + CHG) / KW);
+    for (; s0 < s_end; s0 += P) {
+      qmm_static_for<P>([&](auto hc) {
+        constexpr int p = hc;
+        const int s = s0 + hc;
+        const int gs = s * KW + kw;
+        store_w(qmm_const<p>{});
+        // The loads of step s + P go out in pieces between the sub-steps of the
+        // math (the wave would otherwise sit in front of the busy address unit for
+        // the whole burst); every path issues all of them, in the same order.
+        auto issue = [&](auto tc) __attribute__((always_inline)) {
+          constexpr int t = tc;
+          load_range(qmm_const<p>{}, s + P, qmm_const<t * 8 / SUB>{}, qmm_const<(t + 1) * 8 / SUB>{});
+        };
+        // (the half trip past an odd number of steps has every sub-step beyond K:
+        // it issues its loads and computes nothing)
+        compute(min(gs - c0, nst - 1), s, issue);
+      });
+    }
   }
 
   // ---- reduction over k-splits, final rounding, store ------------------------------------
@@ -544,12 +592,13 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
     static thread_local bool attr_set = false;
     if (!attr_set) {
       int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 Cfg::LDS_BYTES), "weight_only_skinny hipFuncSetAttribute");
+                                                 Cfg::lds_bytes(Cfg::CHG)), "weight_only_skinny hipFuncSetAttribute");
       if (rc != XLA_AMD_QMM_OK) return rc;
       attr_set = true;
     }
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWaves * 64), Cfg::LDS_BYTES, stream, a);
+    const int steps = (a.K + Cfg::KS - 1) / Cfg::KS;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWaves * 64), Cfg::lds_bytes(steps), stream, a);
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
