@@ -81,6 +81,22 @@ __device__ __forceinline__ float qmm_round_dt(float f, int dt) {
   return f;
 }
 
+// Element i as raw bits, without a branch on the dtype and without touching the
+// value: a prefetch written with qmm_load would wait for each element in turn
+// (the conversion sits inside the dtype branch).  qmm_from_raw converts later.
+__device__ __forceinline__ uint32_t qmm_load_raw(const void* p, int64_t i, int dt) {
+  const int esz = dt == XLA_AMD_DT_F32 ? 4 : 2;
+  const char* q = (const char*)p + i * esz;
+  const uint32_t lo = *(const uint16_t*)q;
+  const uint32_t hi = *(const uint16_t*)(q + (esz - 2));  // the same halfword again for 2-byte types
+  return lo | (hi << 16);
+}
+__device__ __forceinline__ float qmm_from_raw(uint32_t raw, int dt) {
+  if (dt == XLA_AMD_DT_BF16) return __uint_as_float(raw << 16);
+  if (dt == XLA_AMD_DT_F16) return qmm_f16_to_f32((uint16_t)(raw & 0xffffu));
+  return __uint_as_float(raw);
+}
+
 __device__ __forceinline__ float qmm_load(const void* p, int64_t i, int dt) {
   if (dt == XLA_AMD_DT_BF16) return qmm_bf16_to_f32(((const uint16_t*)p)[i]);
   if (dt == XLA_AMD_DT_F16) return qmm_f16_to_f32(((const uint16_t*)p)[i]);

@@ -57,8 +57,8 @@ int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t
 
 namespace {
 
-constexpr int kWaves = 4;
-constexpr int kWSeg = 512;        // weight bytes per row per step
+constexpr int kWaves = 4;         // waves per workgroup of the standard shape
+constexpr int kWSeg = 512;        // weight bytes per row per step of the standard shape
 constexpr int kLdsLimit = 160 * 1024;
 
 // ---- operand fragments --------------------------------------------------------
@@ -137,29 +137,33 @@ constexpr int kRedNone = 0;    // blockwise, KW == 1: nothing to reduce
 constexpr int kRedRaw = 1;     // per-channel (C == K, any KW): raw dot products and x sums are summed, then scaled
 constexpr int kRedScaled = 2;  // blockwise, KW > 1, whole blocks per step (KS % C == 0): scaled block results are summed
 
-template <int XT, int BITS, int MT, int KW>
+// NW waves per workgroup; WSEG weight bytes per row per step.
+template <int XT, int BITS, int MT, int KW, int NW = kWaves, int WSEG = kWSeg>
 struct SkinnyCfg {
-  static constexpr int RW = kWaves / KW;
+  static constexpr int RW = NW / KW;
   static constexpr int XB = XT == XLA_AMD_DT_F32 ? 4 : 2;
-  static constexpr int KS = BITS == 8 ? kWSeg : 2 * kWSeg;  // columns per step
+  static constexpr int KS = BITS == 8 ? WSEG : 2 * WSEG;    // columns per step
   static constexpr int SUB = KS / 128;                       // 128-column sub-steps per step
   static constexpr int XROW = KS * XB;                       // bytes of one x row per step
   static constexpr int XROWS = 16 * MT;
-  static constexpr int W_TILE = kWaves * 16 * kWSeg;         // 32 KB: every wave's private 16 rows x 512 B
+  static constexpr int W_TILE = NW * 16 * WSEG;              // 32 KB: every wave's private 16 rows x WSEG bytes
+  static constexpr int NLD = 16 * WSEG / 1024;               // 1 KB weight loads per wave per step
   static constexpr int X_TILE = XROWS * XROW;                // the x columns of one step, all rows
   static constexpr int CH = (kLdsLimit - W_TILE) / X_TILE;   // steps whose x columns are resident in LDS together
-  static constexpr int XPW = X_TILE / 1024 / kWaves;         // 1 KB pieces of an x tile copied by each wave
+  static constexpr int XPW = X_TILE / 1024 / NW;             // 1 KB pieces of an x tile copied by each wave
   static constexpr int P = 2;                                // steps of weight loads in flight (register ring)
   static constexpr int CHG = CH / (2 * KW) * (2 * KW);       // ... rounded so that a chunk holds an even number of steps of every wave
   static constexpr bool kFits = CHG >= 2 * KW;
   static constexpr int lds_bytes(int steps) { return W_TILE + (steps < CHG ? steps : CHG) * X_TILE; }
-  static_assert((X_TILE / 1024) % kWaves == 0, "x tile must split evenly over the waves");
+  static_assert((X_TILE / 1024) % NW == 0, "x tile must split evenly over the waves");
+  static_assert(WSEG == 512 || (WSEG == 256 && BITS == 8), "weight segment");
 };
 
-template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
-__global__ void __launch_bounds__(kWaves * 64)
+template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, int NW = kWaves, int WSEG = kWSeg>
+__global__ void __launch_bounds__(NW * 64)
 qmm_skinny_kernel(SkinnyArgs a) {
-  using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
+  using Cfg = SkinnyCfg<XT, BITS, MT, KW, NW, WSEG>;
+  constexpr int NLD = Cfg::NLD;
   constexpr int RW = Cfg::RW, XB = Cfg::XB, KS = Cfg::KS, SUB = Cfg::SUB, XROW = Cfg::XROW;
   constexpr int W_TILE = Cfg::W_TILE, X_TILE = Cfg::X_TILE, XPW = Cfg::XPW, P = Cfg::P;
   constexpr bool kMfma = XT != XLA_AMD_DT_F32;
@@ -180,59 +184,64 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // ---- global -> register loads (coalesced) ------------------------------------
   // Addresses are a workgroup-uniform base (scalar registers, advanced per step
   // with scalar arithmetic) plus a per-lane 32-bit offset that never changes.
-  // weights: instruction i covers rows 2i, 2i+1 of the wave's 16, 512 B each
+  // weights: instruction i covers 1024 / WSEG consecutive rows of the wave's 16, WSEG bytes each
   const int n_wg = blockIdx.x * (16 * RW);
   const uint8_t* const w_base = a.w + (size_t)n_wg * row_bytes;
   const char* const x_base = (const char*)a.x;
-  const int w_lrow = lane >> 5, w_chunk = lane & 31;
-  uint32_t w_off[8];
-  int w_dst[8];
-  qmm_static_for<8>([&](auto ic) {
+  constexpr int kChunksPerSeg = WSEG / 16;
+  const int w_lrow = lane / kChunksPerSeg, w_chunk = lane % kChunksPerSeg;
+  uint32_t w_off[NLD];
+  int w_dst[NLD];
+  qmm_static_for<NLD>([&](auto ic) {
     constexpr int i = ic;
-    const int row = 2 * i + w_lrow;
+    const int row = (1024 / WSEG) * i + w_lrow;
     const int n = min(n_wave + row, N - 1);  // tail rows read the last valid row
     w_off[i] = (uint32_t)(n - n_wg) * (uint32_t)row_bytes + w_chunk * 16;
-    w_dst[i] = wave * (16 * kWSeg) + row * kWSeg + ((w_chunk ^ row) * 16);
+    w_dst[i] = wave * (16 * WSEG) + row * WSEG + ((w_chunk ^ row) * 16);
   });
   // x: copied global -> LDS without passing registers (global_load_lds_dwordx4:
   // lane l of an instruction lands at base + 16 l).  Piece j of this wave is
-  // 1 KB of one row of a step's tile; the XOR swizzle of the tile is applied on
-  // the source side: LDS slot c' of a row receives global chunk c' ^ (row % 16).
+  // 1 KB of a step's tile: part of one row, or whole consecutive rows when a row
+  // is shorter.  The XOR swizzle of the tile is applied on the source side: LDS
+  // slot c' of a row receives global chunk c' ^ (row % 16).
+  constexpr int kPiecesPerRow = XROW >= 1024 ? XROW / 1024 : 1;
+  constexpr int kRowsPerPiece = XROW >= 1024 ? 1 : 1024 / XROW;
+  constexpr int kLanesPerRow = 64 / kRowsPerPiece;
   uint32_t x_off[XPW];  // per lane: byte offset of its source chunk from the step's first column of row 0
   int x_col[XPW];       // per lane: byte column of that chunk within the step
   int x_lds[XPW];       // uniform: LDS offset of the piece within a tile
   qmm_static_for<XPW>([&](auto jc) {
     constexpr int j = jc;
-    constexpr int kPiecesPerRow = XROW / 1024;
     const int q = wave * XPW + j;
-    const int row = q / kPiecesPerRow, piece = q % kPiecesPerRow;
+    const int row0 = (q / kPiecesPerRow) * kRowsPerPiece, piece = q % kPiecesPerRow;
+    const int row = row0 + lane / kLanesPerRow;
     const int m = min(row, M - 1);
-    x_col[j] = (piece * 64 + (lane ^ (row & 15))) * 16;
+    x_col[j] = ((piece * 64 + lane % kLanesPerRow) ^ (row & 15)) * 16;
     x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + x_col[j];
-    x_lds[j] = W_TILE + row * XROW + piece * 1024;
+    x_lds[j] = W_TILE + row0 * XROW + piece * 1024;
   });
 
   const int steps_total = (K + KS - 1) / KS;
   const int my_steps = steps_total > kw ? (steps_total - kw + KW - 1) / KW : 0;
 
-  i32x4 wreg[P][8];
-  // Weight loads number lo..hi-1 of a step's 8 into ring slot p.
+  i32x4 wreg[P][NLD];
+  // Weight loads number lo..hi-1 of a step's NLD into ring slot p.
   auto load_range = [&](auto pc, int s, auto loc, auto hic) __attribute__((always_inline)) {  // s: this wave's s-th step
     constexpr int p = pc, lo = loc, hi = hic;
     // global step; steps past the end (issued only to keep the number of
     // outstanding loads the same on every path) re-read the last real step
     const int gs = min(s * KW + kw, steps_total - 1);
-    const uint8_t* const wp = w_base + (size_t)gs * kWSeg;
+    const uint8_t* const wp = w_base + (size_t)gs * WSEG;
     if ((gs + 1) * KS <= K) {  // whole step inside K: no per-lane conditions
-      qmm_static_for<8>([&](auto ic) {
+      qmm_static_for<NLD>([&](auto ic) {
         constexpr int i = ic;
         if constexpr (i >= lo && i < hi) wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
       });
     } else {
       // last, partial step: columns past K re-read the last valid 16 bytes of the
       // row (their sub-steps are never computed)
-      const int w_left = row_bytes - gs * kWSeg;
-      qmm_static_for<8>([&](auto ic) {
+      const int w_left = row_bytes - gs * WSEG;
+      qmm_static_for<NLD>([&](auto ic) {
         constexpr int i = ic;
         if constexpr (i >= lo && i < hi) {
           // w_left >= 64 here, so 0 <= back <= w_chunk * 16 <= w_off[i]
@@ -243,7 +252,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
     }
   };
   auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {
-    load_range(pc, s, qmm_const<0>{}, qmm_const<8>{});
+    load_range(pc, s, qmm_const<0>{}, qmm_const<NLD>{});
   };
   // The x columns of global steps c0 .. c0+nst-1 into the LDS tiles 0 .. nst-1.
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -274,7 +283,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // a second stage nor a barrier is needed around it.
   auto store_w = [&](auto pc) __attribute__((always_inline)) {
     constexpr int p = pc;
-    qmm_static_for<8>([&](auto ic) {
+    qmm_static_for<NLD>([&](auto ic) {
       constexpr int i = ic;
       *(i32x4*)(smem + w_dst[i]) = wreg[p][i];
     });
@@ -305,13 +314,13 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // zacc += round_x(xsum) * zp[s,n]; the block accumulators restart.
   // Per-channel: the only scales a lane ever needs are fetched now, so that
   // their latency is hidden behind the main loop instead of trailing it.
-  float pre_sc[4] = {0.f, 0.f, 0.f, 0.f}, pre_zp[4] = {0.f, 0.f, 0.f, 0.f};
+  uint32_t pre_sc[4] = {0u, 0u, 0u, 0u}, pre_zp[4] = {0u, 0u, 0u, 0u};  // raw bits: converted where they are used
   if constexpr (RED == kRedRaw) {
     qmm_static_for<4>([&](auto vc) {
       constexpr int v = vc;
       const int n = min(n_wave + 4 * g + v, N - 1);
-      pre_sc[v] = qmm_load(a.scale, n, a.scale_dt);
-      if constexpr (HASZP) pre_zp[v] = qmm_load(a.zp, n, a.zp_dt);
+      pre_sc[v] = qmm_load_raw(a.scale, n, a.scale_dt);
+      if constexpr (HASZP) pre_zp[v] = qmm_load_raw(a.zp, n, a.zp_dt);
     });
   }
   auto block_epilogue = [&](int sblk) __attribute__((always_inline)) {
@@ -320,8 +329,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
       const int n = min(n_wave + 4 * g + v, N - 1);
       float sc, zv = 0.f;
       if constexpr (RED == kRedRaw) {
-        sc = pre_sc[v];
-        zv = pre_zp[v];
+        sc = qmm_from_raw(pre_sc[v], a.scale_dt);
+        if constexpr (HASZP) zv = qmm_from_raw(pre_zp[v], a.zp_dt);
       } else {
         sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
         if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
@@ -351,7 +360,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // beyond K are skipped (a uniform branch around arithmetic only: the loads stay
   // in straight-line code, so the compiler's wait counts for the ring stay exact).
   auto compute = [&](int tile, int s, auto&& issue) __attribute__((always_inline)) {
-    const char* wb = smem + wave * (16 * kWSeg) + r * kWSeg;
+    const char* wb = smem + wave * (16 * WSEG) + r * WSEG;
     const char* xb = smem + W_TILE + tile * X_TILE;
     const int k_step = (s * KW + kw) * KS;
     if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
@@ -492,7 +501,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
         // the whole burst); every path issues all of them, in the same order.
         auto issue = [&](auto tc) __attribute__((always_inline)) {
           constexpr int t = tc;
-          load_range(qmm_const<p>{}, s + P, qmm_const<t * 8 / SUB>{}, qmm_const<(t + 1) * 8 / SUB>{});
+          load_range(qmm_const<p>{}, s + P, qmm_const<t * NLD / SUB>{}, qmm_const<(t + 1) * NLD / SUB>{});
         };
         // (the half trip past an odd number of steps has every sub-step beyond K:
         // it issues its loads and computes nothing)
@@ -582,13 +591,13 @@ qmm_skinny_kernel(SkinnyArgs a) {
   });
 }
 
-template <int XT, int BITS, int MT, int KW, int RED, bool HASZP>
+template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, int NW = kWaves, int WSEG = kWSeg>
 int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
-  using Cfg = SkinnyCfg<XT, BITS, MT, KW>;
+  using Cfg = SkinnyCfg<XT, BITS, MT, KW, NW, WSEG>;
   if constexpr (!Cfg::kFits) {
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: tile does not fit in LDS");
   } else {
-    auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP>;
+    auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, NW, WSEG>;
     static thread_local bool attr_set = false;
     if (!attr_set) {
       int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -598,7 +607,7 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
     }
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
     const int steps = (a.K + Cfg::KS - 1) / Cfg::KS;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(kWaves * 64), Cfg::lds_bytes(steps), stream, a);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NW * 64), Cfg::lds_bytes(steps), stream, a);
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
@@ -623,8 +632,17 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
     if (a.N < 200 * 64 && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
     if (a.N < 200 * 32 && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
   }
-  if (kw == 1) return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
-                            : launch_zp<XT, BITS, MT, 1, kRedNone>(a, haszp, stream);
+  if (kw == 1) {
+    // Large N, per-channel int8, up to 16 rows: 8 waves per workgroup (two per
+    // SIMD, so that one wave's waits are another's issue slots) as 4 row groups
+    // x 2 k-splits, walking K in steps of 256 columns.
+    if constexpr (BITS == 8 && MT == 1 && XT != XLA_AMD_DT_F32) {
+      if (perch) return haszp ? launch_kernel<XT, 8, 1, 2, kRedRaw, true, 8, 256>(a, stream)
+                              : launch_kernel<XT, 8, 1, 2, kRedRaw, false, 8, 256>(a, stream);
+    }
+    return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
+                 : launch_zp<XT, BITS, MT, 1, kRedNone>(a, haszp, stream);
+  }
   if (kw == 2) return perch ? launch_zp<XT, BITS, MT, 2, kRedRaw>(a, haszp, stream)
                             : launch_zp<XT, BITS, MT, 2, kRedScaled>(a, haszp, stream);
   return perch ? launch_zp<XT, BITS, MT, 4, kRedRaw>(a, haszp, stream)

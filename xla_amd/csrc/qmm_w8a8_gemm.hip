@@ -142,17 +142,18 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   static_assert(BM <= T && BN <= T, "one scale per thread");
   const bool has_zp = g.zp != nullptr;
   const bool want_out = g.out != nullptr, want_acc = g.acc_out != nullptr;
-  float pre_xs = 0.f, pre_xsum = 0.f, pre_ws = 0.f, pre_zp = 0.f;
+  // (raw bits, loaded without a branch on the dtype: converting here would make
+  // the kernel wait for each of these loads in turn before its first copy)
+  uint32_t pre_xs = 0u, pre_ws = 0u, pre_zp = 0u;
+  int pre_xsum = 0;
   if (want_out) {
-    if (tid < BM) {
-      const int m = min(m0 + tid, g.M - 1);
-      pre_xs = qmm_load(g.x_scale, m, g.x_scale_dt);
-      if (has_zp) pre_xsum = qmm_round_dt((float)g.x_sum[m], g.zpo_dt);
-    }
-    if (tid < BN) {
-      const int n = min(n0 + tid, g.N - 1);
-      pre_ws = qmm_load(g.w_scale, n, g.w_scale_dt);
-      if (has_zp) pre_zp = qmm_load(g.zp, n, g.zp_dt);
+    const int m = min(m0 + min(tid, BM - 1), g.M - 1);
+    const int n = min(n0 + min(tid, BN - 1), g.N - 1);
+    pre_xs = qmm_load_raw(g.x_scale, m, g.x_scale_dt);
+    pre_ws = qmm_load_raw(g.w_scale, n, g.w_scale_dt);
+    if (has_zp) {
+      pre_xsum = g.x_sum[m];
+      pre_zp = qmm_load_raw(g.zp, n, g.zp_dt);
     }
   }
 
@@ -231,8 +232,14 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   float* s_ws = s_xsum + BM;           // [BN] weight scale
   float* s_zp = s_ws + BN;             // [BN] zero point
   int* s_ep = (int*)(s_zp + BN) + wave * (32 * kEpStride);  // per-wave [32][kEpStride]
-  if (tid < BM) { s_xs[tid] = pre_xs; s_xsum[tid] = pre_xsum; }
-  if (tid < BN) { s_ws[tid] = pre_ws; s_zp[tid] = pre_zp; }
+  if (tid < BM) {
+    s_xs[tid] = qmm_from_raw(pre_xs, g.x_scale_dt);
+    s_xsum[tid] = has_zp ? qmm_round_dt((float)pre_xsum, g.zpo_dt) : 0.f;
+  }
+  if (tid < BN) {
+    s_ws[tid] = qmm_from_raw(pre_ws, g.w_scale_dt);
+    s_zp[tid] = has_zp ? qmm_from_raw(pre_zp, g.zp_dt) : 0.f;
+  }
   __syncthreads();
   constexpr int kLanesPerRow = TN / 4;               // each lane finishes 4 consecutive n
   constexpr int kPasses = 32 * kLanesPerRow / 64;    // passes over a 32-row block
