@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define XLA_AMD_QMM_ABI_VERSION 1
+#define XLA_AMD_QMM_ABI_VERSION 2
 
 /* return codes */
 #define XLA_AMD_QMM_OK 0
@@ -72,8 +72,8 @@ const char* xla_amd_qmm_last_error(void);
 size_t xla_amd_qmm_packed_bytes(int64_t N, int64_t K, int bits);
 
 /*
- * One-time re-layout of a weight into the K-major form the streaming kernel
- * reads.  Replaces the reference's `_xla_cast_int4(w, w.cpu()...tolist())`
+ * One-time re-layout of a weight into plain K-major form (rows of K values;
+ * for bits == 4 two values per byte).  Replaces the reference's `_xla_cast_int4(w, w.cpu()...tolist())`
  * (xla_quantized_matmul.py:101-103 -> csrc/ops/cast_int4.cpp:30-39), which
  * rebuilds the weight as an s4 literal: values are unchanged, only storage.
  *   src_layout XLA_AMD_W_NK : w is [N, K]       (C ignored, S*C == K)
@@ -88,19 +88,43 @@ int xla_amd_qmm_pack_weight(const int8_t* w, void* packed, int64_t S, int64_t C,
                             int src_layout, int bits, void* stream);
 
 /*
- * Weight-only quantized matmul, fast path: streams a K-major weight once and
- * keeps up to 64 rows of x per pass in MFMA fragments (passes over w repeat
+ * Bytes of the tiled copy of a weight that the streaming kernel reads:
+ * ceil(N/16)*16 * K for bits == 8, half of that for bits == 4.  Needs
+ * K % 128 == 0; returns 0 for arguments the tile kernel rejects.
+ */
+size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits);
+
+/*
+ * One-time re-layout of a weight into the tiled form the streaming kernel
+ * reads (same arguments and the same reference statement as
+ * xla_amd_qmm_pack_weight: values are unchanged, only storage).  Needs
+ * K % 128 == 0.  For every group g of 16 consecutive channels and every
+ * sub-step t of 128 consecutive columns there is one block of BLK bytes at
+ * byte offset (g * (K/128) + t) * BLK; channels past N are stored as zero.
+ *   bits 8 (BLK 2048): byte h*1024 + l*16 + j (h in 0..1, l in 0..63, j in 0..15)
+ *           holds w(16g + l%16, 128t + 32*(l/16) + 16h + j).
+ *   bits 4 (BLK 1024): the 32-bit word at byte l*16 + 4i (i in 0..3) holds the
+ *           8 columns 128t + 32*(l/16) + 8i .. +7 of channel 16g + l%16 in the
+ *           nibble order of xla_amd_qmm_pack_weight.
+ * A 64-lane load of 16 bytes per lane from consecutive addresses thus puts
+ * into lane l exactly the MFMA operand fragment of channel l%16.
+ */
+int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, int64_t N,
+                            int src_layout, int bits, void* stream);
+
+/*
+ * Weight-only quantized matmul, fast path: streams a tiled weight once and
+ * keeps up to 32 rows of x per pass in MFMA fragments (passes over w repeat
  * for larger M).  Replaces, with the reference's rounding points,
  *   per-channel (C == K):  out = F.linear(x, w) * scaler      (:113-114)
  *   blockwise   (C <  K):  einsum('scn,...sc->...sn'), einsum('sn,...sn->...n') (:122-124)
  *   zero point:            out -= rowsum/blocksum(x) (x) zp    (:125-133)
- * x [M,K] (bf16/f16/f32), w_packed from xla_amd_qmm_pack_weight (a per-channel
- * int8 [N,K] weight already is its own 8-bit packed form), scale [S,N],
+ * x [M,K] (bf16/f16/f32), w_tiled from xla_amd_qmm_tile_weight, scale [S,N],
  * zp [S,N] or NULL, out [M,N].
  * Needs K % 128 == 0 and C % 128 == 0; else XLA_AMD_QMM_EUNSUPPORTED.
  * out_dt must be the torch promotion of (x_dt, scale_dt).
  */
-int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packed, const void* scale,
+int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const void* scale,
                                    const void* zp, void* out, int64_t M, int64_t N, int64_t K,
                                    int64_t C, int bits, int x_dt, int scale_dt, int zp_dt,
                                    int out_dt, void* stream);

@@ -289,6 +289,42 @@ def test_golden_dot_general_and_int4_pack(ops):
     assert packed.tolist() == [r["word"] for r in rows]
 
 
+def test_tile_weight_layout(ops):
+  # the tiled copy against its written definition (include/xla_amd_qmm.h), both source layouts, N tail
+  from xla_amd import _lib
+  n, k = 40, 256
+  g = cases.gen(7)
+  for bits in (8, 4):
+    lo, hi = (-128, 128) if bits == 8 else (-8, 8)
+    w = torch.randint(lo, hi, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+    wn = w.numpy().astype(np.int64)
+    groups, n_blk = (n + 15) // 16, k // 128
+    blk = 2048 if bits == 8 else 1024
+    expect = np.zeros(groups * n_blk * blk, dtype=np.uint8)
+    P = [0, 2, 4, 6, 1, 3, 5, 7]
+    for gi in range(groups):
+      for t in range(n_blk):
+        base = (gi * n_blk + t) * blk
+        for l in range(64):
+          ch, k0 = 16 * gi + l % 16, 128 * t + 32 * (l // 16)
+          if ch >= n:
+            continue
+          if bits == 8:
+            for h in range(2):
+              for j in range(16):
+                expect[base + h * 1024 + l * 16 + j] = wn[ch, k0 + 16 * h + j] & 0xFF
+          else:
+            for i in range(4):
+              word = 0
+              for j in range(8):
+                word |= ((int(wn[ch, k0 + 8 * i + P[j]]) + 8) & 15) << (4 * j)
+              for b in range(4):
+                expect[base + l * 16 + 4 * i + b] = (word >> (8 * b)) & 0xFF
+    for layout, src in ((_lib.W_NK, w), (_lib.W_SCN, w.T.reshape(2, 128, n).contiguous())):
+      got = ops._tiled_weight(src.cuda(), bits, layout).cpu().numpy()
+      assert got.shape == expect.shape and np.array_equal(got, expect), (bits, layout)
+
+
 def test_w8a8_tiles_and_tails(ops):
   # every workgroup tile the kernel offers, on shapes with M/N/K tails
   for bm in (64, 128, 256):

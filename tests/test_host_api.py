@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
   for n in names:
     assert hasattr(lib, n), f"{n} declared in the header but not exported"
   assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-  assert lib.xla_amd_qmm_abi_version() == 1
+  assert lib.xla_amd_qmm_abi_version() == 2
 
 
 def test_header_cites_reference_for_each_entry_point():
@@ -65,6 +65,9 @@ def test_error_codes_without_gpu():
   assert lib.xla_amd_qmm_packed_bytes(8, 64, 8) == 512
   assert lib.xla_amd_qmm_packed_bytes(8, 64, 4) == 256
   assert lib.xla_amd_qmm_packed_bytes(8, 5, 4) == 0
+  assert lib.xla_amd_qmm_tiled_bytes(17, 256, 8) == 32 * 256
+  assert lib.xla_amd_qmm_tiled_bytes(16, 128, 4) == 16 * 64
+  assert lib.xla_amd_qmm_tiled_bytes(16, 64, 8) == 0
   rc = lib.xla_amd_qmm_weight_only_skinny(None, None, None, None, None, 1, 1, 128, 128, 8, 1, 1, 1, 1, None)
   assert rc == _lib.EINVAL and b"null" in lib.xla_amd_qmm_last_error()
   rc = lib.xla_amd_qmm_quantize_per_token(None, None, None, None, 1, 1, 0, 0, 0, None)

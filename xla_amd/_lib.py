@@ -16,7 +16,7 @@ DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 OVERFLOW_SATURATE, OVERFLOW_WRAP = 0, 1
 W_NK, W_SCN = 0, 1
 KERNEL_GENERIC, KERNEL_SKINNY_MFMA, KERNEL_W8A8_MFMA, KERNEL_W8A8_GENERIC = 0, 1, 2, 3
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 
@@ -28,6 +28,8 @@ SIGNATURES = {
     "xla_amd_qmm_last_error": (ctypes.c_char_p, []),
     "xla_amd_qmm_packed_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_int]),
     "xla_amd_qmm_pack_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
+    "xla_amd_qmm_tiled_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_int]),
+    "xla_amd_qmm_tile_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
     "xla_amd_qmm_weight_only_skinny": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 5 + [_c_vp]),
     "xla_amd_qmm_weight_only_generic": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 5 + [_c_vp]),
     "xla_amd_qmm_quantize_per_token": (_c_int, [_c_vp] * 4 + [_c_i64] * 2 + [_c_int] * 3 + [_c_vp]),

@@ -30,6 +30,12 @@ extern "C" size_t xla_amd_qmm_packed_bytes(int64_t N, int64_t K, int bits) {
   return 0;
 }
 
+extern "C" size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits) {
+  if (N <= 0 || K <= 0 || K % 128 != 0 || (bits != 4 && bits != 8)) return 0;
+  const size_t rows = (size_t)((N + 15) / 16) * 16;
+  return bits == 8 ? rows * (size_t)K : rows * (size_t)K / 2;
+}
+
 // The two regimes of a quantized linear layer on MI355X:
 //  * few rows of x (decode): every weight byte is used M times, far below the
 //    ~630 int8 ops/byte (or ~310 bf16 flops/byte) the chip can do per HBM

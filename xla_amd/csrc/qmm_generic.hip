@@ -147,6 +147,59 @@ qmm_pack_kernel(const int8_t* __restrict__ w, uint32_t* __restrict__ packed, int
   packed[n * words_per_row + g] = word;
 }
 
+// Tiled copy for the streaming kernel: one thread writes the 16 bytes that one
+// lane of one 1 KB load will receive.
+__global__ void __launch_bounds__(256)
+qmm_tile_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ tiled, int64_t N, int64_t K,
+                int src_layout, int bits, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int chunks = bits == 8 ? 128 : 64;  // 16-byte chunks per block
+  const int c = (int)(idx % chunks);
+  const int64_t blk = idx / chunks;
+  const int64_t n_blk = K / 128;
+  const int64_t t = blk % n_blk, g = blk / n_blk;
+  const int l = c & 63, h = c >> 6;
+  const int64_t n = 16 * g + (l & 15);
+  const int64_t k0 = 128 * t + 32 * (l >> 4) + 16 * h;
+  auto at = [&](int64_t k) -> int { return src_layout == XLA_AMD_W_NK ? w[n * K + k] : w[k * N + n]; };
+  i32x4 v = {0, 0, 0, 0};
+  if (n < N) {
+    if (bits == 8) {
+      for (int i = 0; i < 4; ++i) {
+        uint32_t word = 0;
+        for (int j = 0; j < 4; ++j) word |= ((uint32_t)(uint8_t)at(k0 + 4 * i + j)) << (8 * j);
+        v[i] = (int)word;
+      }
+    } else {
+      const int P[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+      for (int i = 0; i < 4; ++i) {
+        uint32_t word = 0;
+        for (int j = 0; j < 8; ++j) word |= ((uint32_t)((at(k0 + 8 * i + P[j]) + 8) & 15)) << (4 * j);
+        v[i] = (int)word;
+      }
+    }
+  }
+  tiled[idx] = v;
+}
+
+extern "C" int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, int64_t N,
+                                       int src_layout, int bits, void* stream) {
+  if (!w || !tiled) return qmm_fail(XLA_AMD_QMM_EINVAL, "tile_weight: null pointer");
+  if (S <= 0 || C <= 0 || N <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "tile_weight: bad sizes");
+  if (bits != 4 && bits != 8) return qmm_fail(XLA_AMD_QMM_EINVAL, "tile_weight: bits must be 4 or 8");
+  if (src_layout != XLA_AMD_W_NK && src_layout != XLA_AMD_W_SCN)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "tile_weight: bad layout %d", src_layout);
+  const int64_t K = S * C;
+  if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "tile_weight: K=%lld not a multiple of 128", (long long)K);
+  const int64_t total = ((N + 15) / 16) * (K / 128) * (bits == 8 ? 128 : 64);
+  const int64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffLL) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "tile_weight: weight too large");
+  hipLaunchKernelGGL(qmm_tile_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, w,
+                     (i32x4*)tiled, N, K, src_layout, bits, total);
+  return QMM_CHECK_LAUNCH("tile_weight launch");
+}
+
 extern "C" int xla_amd_qmm_pack_weight(const int8_t* w, void* packed, int64_t S, int64_t C, int64_t N,
                                        int src_layout, int bits, void* stream) {
   if (!w || !packed) return qmm_fail(XLA_AMD_QMM_EINVAL, "pack_weight: null pointer");

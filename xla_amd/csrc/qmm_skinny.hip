@@ -1,15 +1,16 @@
 // Weight-streaming GEMV / skinny GEMM for weight-only quantized linear layers
 // on gfx950.  HBM-bound: every weight byte is read from memory exactly once.
 //
-// Memory access.  Weight loads are issued so that one wave instruction reads
-// long contiguous runs (2 weight rows x 512 B): that is what the memory system
-// streams fastest.  The matrix cores want the opposite arrangement (lane = row,
-// 8 consecutive k per lane), so a wave's weights take one trip through its own
-// LDS tile: written as they were loaded, read back in MFMA operand order.
-// 16-byte chunks are XOR-swizzled with the row number so that both directions
-// are free of bank conflicts.  The activations are copied global -> LDS without
-// passing registers, a chunk of up to 128 KB of x columns at a time (all of x
-// for 16 rows x 4096 bf16 columns), and stay there while the weights stream by.
+// Memory access.  The weights are read from a tiled copy made once per weight
+// (xla_amd_qmm_tile_weight): for every 16 channels x 128 columns one block
+// whose bytes are already in MFMA operand order (lane = channel, 32 consecutive
+// k per lane), blocks of a channel group consecutive along K.  A wave therefore
+// streams one contiguous region with 1 KB loads that land directly in operand
+// registers: no transposition, no LDS traffic for weights.  The activations are
+// copied global -> LDS without passing registers, a chunk of up to 160 KB of x
+// columns at a time (all of x for 16 rows x 4096 bf16 columns), XOR-swizzled so
+// that the operand reads are free of bank conflicts, and stay there while the
+// weights stream by.
 //
 // Work split.  A workgroup has 4 waves arranged as RW row groups x KW k-splits
 // (RW * KW == 4).  It owns 16*RW consecutive output channels.  K is walked in
@@ -21,7 +22,7 @@
 // Synchronisation.  The workgroup meets only when the resident x columns are
 // replaced.  In between nothing is shared but read-only x, so every wave runs
 // at its own pace: wait for its weight loads (a ring of two steps in flight,
-// re-issued piecewise between the multiplies), transpose, multiply.  The waves
+// re-issued piecewise between the multiplies), multiply.  The waves
 // of a compute unit drift apart, and the memory waits of one overlap the LDS
 // traffic and arithmetic of the others; a barrier per step would instead make
 // each step as slow as its slowest wave.
@@ -146,15 +147,19 @@ struct SkinnyCfg {
   static constexpr int SUB = KS / 128;                       // 128-column sub-steps per step
   static constexpr int XROW = KS * XB;                       // bytes of one x row per step
   static constexpr int XROWS = 16 * MT;
-  static constexpr int W_TILE = NW * 16 * WSEG;              // 32 KB: every wave's private 16 rows x WSEG bytes
   static constexpr int NLD = 16 * WSEG / 1024;               // 1 KB weight loads per wave per step
+  static constexpr int BLK = BITS == 8 ? 2048 : 1024;        // bytes of one (16 channels x 128 columns) weight block
   static constexpr int X_TILE = XROWS * XROW;                // the x columns of one step, all rows
-  static constexpr int CH = (kLdsLimit - W_TILE) / X_TILE;   // steps whose x columns are resident in LDS together
+  static constexpr int CH = kLdsLimit / X_TILE;              // steps whose x columns are resident in LDS together
   static constexpr int XPW = X_TILE / 1024 / NW;             // 1 KB pieces of an x tile copied by each wave
   static constexpr int P = 2;                                // steps of weight loads in flight (register ring)
   static constexpr int CHG = CH / (2 * KW) * (2 * KW);       // ... rounded so that a chunk holds an even number of steps of every wave
   static constexpr bool kFits = CHG >= 2 * KW;
-  static constexpr int lds_bytes(int steps) { return W_TILE + (steps < CHG ? steps : CHG) * X_TILE; }
+  static constexpr int kRedBytes = NW * 16 * MT * 256;       // cross-wave reduction scratch (reuses the x tiles)
+  static constexpr int lds_bytes(int steps) {
+    const int x = (steps < CHG ? steps : CHG) * X_TILE;
+    return x > kRedBytes ? x : kRedBytes;
+  }
   static_assert((X_TILE / 1024) % NW == 0, "x tile must split evenly over the waves");
   static_assert(WSEG == 512 || (WSEG == 256 && BITS == 8), "weight segment");
 };
@@ -165,7 +170,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   using Cfg = SkinnyCfg<XT, BITS, MT, KW, NW, WSEG>;
   constexpr int NLD = Cfg::NLD;
   constexpr int RW = Cfg::RW, XB = Cfg::XB, KS = Cfg::KS, SUB = Cfg::SUB, XROW = Cfg::XROW;
-  constexpr int W_TILE = Cfg::W_TILE, X_TILE = Cfg::X_TILE, XPW = Cfg::XPW, P = Cfg::P;
+  constexpr int X_TILE = Cfg::X_TILE, XPW = Cfg::XPW, P = Cfg::P, BLK = Cfg::BLK;
   constexpr bool kMfma = XT != XLA_AMD_DT_F32;
   constexpr bool NEEDXS = HASZP || (BITS == 4 && kMfma);  // x sums: zero point, int4 affine map
   constexpr int XQ = kMfma ? 4 : 8;                       // 16-byte x chunks per lane per sub-step
@@ -178,27 +183,18 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int r = lane & 15, g = lane >> 4;
   const int K = a.K, N = a.N, M = a.M, C = a.C;
   const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
-  const int row_bytes = BITS == 8 ? K : K / 2;          // bytes of one weight row
   const int x_dt = XT;
 
-  // ---- global -> register loads (coalesced) ------------------------------------
-  // Addresses are a workgroup-uniform base (scalar registers, advanced per step
-  // with scalar arithmetic) plus a per-lane 32-bit offset that never changes.
-  // weights: instruction i covers 1024 / WSEG consecutive rows of the wave's 16, WSEG bytes each
-  const int n_wg = blockIdx.x * (16 * RW);
-  const uint8_t* const w_base = a.w + (size_t)n_wg * row_bytes;
+  // ---- weights: global -> registers, already in MFMA operand order ------------------
+  // The tiled weight holds, for every group of 16 channels and every sub-step of
+  // 128 columns, one block of BLK bytes; the blocks of a group follow each other
+  // along K, so a wave streams one contiguous region.  Lane l of a 1 KB load
+  // takes bytes [16 l, 16 l + 16): its own operand fragment.
+  const int n_blk = K / 128;                                    // blocks per channel group
+  const int groups = (N + 15) / 16;
+  const int my_group = min((int)blockIdx.x * RW + rw, groups - 1);  // tail groups re-read the last one
+  const uint8_t* const w_base = a.w + (size_t)my_group * n_blk * BLK + lane * 16;
   const char* const x_base = (const char*)a.x;
-  constexpr int kChunksPerSeg = WSEG / 16;
-  const int w_lrow = lane / kChunksPerSeg, w_chunk = lane % kChunksPerSeg;
-  uint32_t w_off[NLD];
-  int w_dst[NLD];
-  qmm_static_for<NLD>([&](auto ic) {
-    constexpr int i = ic;
-    const int row = (1024 / WSEG) * i + w_lrow;
-    const int n = min(n_wave + row, N - 1);  // tail rows read the last valid row
-    w_off[i] = (uint32_t)(n - n_wg) * (uint32_t)row_bytes + w_chunk * 16;
-    w_dst[i] = wave * (16 * WSEG) + row * WSEG + ((w_chunk ^ row) * 16);
-  });
   // x: copied global -> LDS without passing registers (global_load_lds_dwordx4:
   // lane l of an instruction lands at base + 16 l).  Piece j of this wave is
   // 1 KB of a step's tile: part of one row, or whole consecutive rows when a row
@@ -218,41 +214,30 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const int m = min(row, M - 1);
     x_col[j] = ((piece * 64 + lane % kLanesPerRow) ^ (row & 15)) * 16;
     x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + x_col[j];
-    x_lds[j] = W_TILE + row0 * XROW + piece * 1024;
+    x_lds[j] = row0 * XROW + piece * 1024;
   });
 
   const int steps_total = (K + KS - 1) / KS;
   const int my_steps = steps_total > kw ? (steps_total - kw + KW - 1) / KW : 0;
 
+  // ring slot p holds the fragments of one step: register 2t + h is half h of
+  // sub-step t (bits 8), register t is sub-step t (bits 4)
   i32x4 wreg[P][NLD];
-  // Weight loads number lo..hi-1 of a step's NLD into ring slot p.
-  auto load_range = [&](auto pc, int s, auto loc, auto hic) __attribute__((always_inline)) {  // s: this wave's s-th step
-    constexpr int p = pc, lo = loc, hi = hic;
-    // global step; steps past the end (issued only to keep the number of
-    // outstanding loads the same on every path) re-read the last real step
-    const int gs = min(s * KW + kw, steps_total - 1);
-    const uint8_t* const wp = w_base + (size_t)gs * WSEG;
-    if ((gs + 1) * KS <= K) {  // whole step inside K: no per-lane conditions
-      qmm_static_for<NLD>([&](auto ic) {
-        constexpr int i = ic;
-        if constexpr (i >= lo && i < hi) wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + w_off[i]));
-      });
-    } else {
-      // last, partial step: columns past K re-read the last valid 16 bytes of the
-      // row (their sub-steps are never computed)
-      const int w_left = row_bytes - gs * WSEG;
-      qmm_static_for<NLD>([&](auto ic) {
-        constexpr int i = ic;
-        if constexpr (i >= lo && i < hi) {
-          // w_left >= 64 here, so 0 <= back <= w_chunk * 16 <= w_off[i]
-          const int back = max(w_chunk * 16 + 16 - w_left, 0);
-          wreg[p][i] = __builtin_nontemporal_load((const i32x4*)(wp + ((int64_t)w_off[i] - back)));
-        }
-      });
-    }
+  constexpr int kLoadsPerSub = NLD / SUB;
+  // The fragments of sub-step t of this wave's s-th step into ring slot p.  Steps
+  // and sub-steps past the end (loaded only to keep the number of outstanding
+  // loads the same on every path) re-read the last block of the group.
+  auto load_sub = [&](auto pc, int s, auto tc) __attribute__((always_inline)) {
+    constexpr int p = pc, t = tc;
+    const int blk = min((s * KW + kw) * SUB + t, n_blk - 1);
+    const uint8_t* const wp = w_base + (size_t)blk * BLK;
+    qmm_static_for<kLoadsPerSub>([&](auto hc) {
+      constexpr int h = hc;
+      wreg[p][kLoadsPerSub * t + h] = __builtin_nontemporal_load((const i32x4*)(wp + h * 1024));
+    });
   };
   auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {
-    load_range(pc, s, qmm_const<0>{}, qmm_const<NLD>{});
+    qmm_static_for<SUB>([&](auto tc) { load_sub(pc, s, tc); });
   };
   // The x columns of global steps c0 .. c0+nst-1 into the LDS tiles 0 .. nst-1.
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -278,17 +263,6 @@ qmm_skinny_kernel(SkinnyArgs a) {
       }
     }
   };
-  // ring slot p -> this wave's private weight tile (swizzled).  Nobody else
-  // touches that tile and a wave's LDS operations execute in order, so neither
-  // a second stage nor a barrier is needed around it.
-  auto store_w = [&](auto pc) __attribute__((always_inline)) {
-    constexpr int p = pc;
-    qmm_static_for<NLD>([&](auto ic) {
-      constexpr int i = ic;
-      *(i32x4*)(smem + w_dst[i]) = wreg[p][i];
-    });
-  };
-
   // ---- accumulators ----------------------------------------------------------------
   // (register arrays are only ever indexed by compile-time constants: every
   // loop over them is a qmm_static_for)
@@ -355,26 +329,20 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // Sub-steps (128 columns) left in the current quantization block; uniform.
   const int sub_per_block = C / 128;
   int block_left = sub_per_block;
-  // issue(t) is called once per sub-step t = 0..SUB-1, before that sub-step's math:
-  // the caller spreads the next loads over the step with it.  Sub-steps at or
-  // beyond K are skipped (a uniform branch around arithmetic only: the loads stay
-  // in straight-line code, so the compiler's wait counts for the ring stay exact).
-  auto compute = [&](int tile, int s, auto&& issue) __attribute__((always_inline)) {
-    const char* wb = smem + wave * (16 * WSEG) + r * WSEG;
-    const char* xb = smem + W_TILE + tile * X_TILE;
+  // One step: the weights of ring slot p against the x columns in LDS tile
+  // `tile`.  As soon as a sub-step's fragments have been used, the same
+  // registers are re-loaded with that sub-step of step s + P: the loads trickle
+  // out between the multiplies instead of as one burst.  Sub-steps at or beyond K
+  // are skipped (a uniform branch around arithmetic only: the loads stay in
+  // straight-line code, so the compiler's wait counts for the ring stay exact).
+  auto compute = [&](auto pc, int tile, int s) __attribute__((always_inline)) {
+    constexpr int p = pc;
+    const char* xb = smem + tile * X_TILE;
     const int k_step = (s * KW + kw) * KS;
     if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
-    // fragments of sub-step t: this lane's 32 weight bytes and, per tile of 16
-    // x rows, its XQ 16-byte chunks of x
-    auto read_frags = [&](auto tc, i32x4& wq0, i32x4& wq1, i32x4 (&xq)[MT][XQ]) __attribute__((always_inline)) {
+    // x fragments of sub-step t: per tile of 16 x rows, this lane's XQ 16-byte chunks
+    auto read_frags = [&](auto tc, i32x4 (&xq)[MT][XQ]) __attribute__((always_inline)) {
       constexpr int t = tc;
-      if constexpr (BITS == 8) {
-        wq0 = *(const i32x4*)(wb + (((8 * t + 2 * g) ^ r) * 16));
-        wq1 = *(const i32x4*)(wb + (((8 * t + 2 * g + 1) ^ r) * 16));
-      } else {
-        wq0 = *(const i32x4*)(wb + (((4 * t + g) ^ r) * 16));
-        wq1 = wq0;
-      }
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
         qmm_static_for<XQ>([&](auto qc) {
@@ -438,29 +406,30 @@ qmm_skinny_kernel(SkinnyArgs a) {
     };
     // (two x tiles with per-block scale accumulators leave no registers for the second fragment set)
     constexpr bool kPipe = kMfma && !(MT == 2 && RED == kRedScaled);
+    constexpr int kW1 = kLoadsPerSub - 1;  // second half of a sub-step's fragment (bits 8), else the same register
     if constexpr (kPipe) {
       // The LDS reads of sub-step t+1 are issued before the math of sub-step t
-      // (a lone wave per SIMD has nobody else to hide LDS latency).
-      i32x4 wq0[2], wq1[2], xq[2][MT][XQ];
-      read_frags(qmm_const<0>{}, wq0[0], wq1[0], xq[0]);
+      // (a wave has few neighbours on its SIMD to hide LDS latency).
+      i32x4 xq[2][MT][XQ];
+      read_frags(qmm_const<0>{}, xq[0]);
       qmm_static_for<SUB>([&](auto tc) {
         constexpr int t = tc;
         constexpr int cur = t & 1, nxt = cur ^ 1;
-        if constexpr (t + 1 < SUB) read_frags(qmm_const<t + 1>{}, wq0[nxt], wq1[nxt], xq[nxt]);
-        issue(tc);
+        if constexpr (t + 1 < SUB) read_frags(qmm_const<t + 1>{}, xq[nxt]);
         __builtin_amdgcn_sched_barrier(0);
-        if (k_step + t * 128 < K) math(tc, wq0[cur], wq1[cur], xq[cur]);
+        if (k_step + t * 128 < K) math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq[cur]);
+        load_sub(pc, s + P, tc);
         __builtin_amdgcn_sched_barrier(0);
       });
     } else {
-      qmm_static_for<SUB>([&](auto tc) { issue(tc); });
       qmm_static_for<SUB>([&](auto tc) {
         constexpr int t = tc;
         if (k_step + t * 128 < K) {
-          i32x4 wq0, wq1, xq[MT][XQ];
-          read_frags(tc, wq0, wq1, xq);
-          math(tc, wq0, wq1, xq);
+          i32x4 xq[MT][XQ];
+          read_frags(tc, xq);
+          math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq);
         }
+        load_sub(pc, s + P, tc);
       });
     }
   };
@@ -468,18 +437,17 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // ---- main loop ---------------------------------------------------------------------
   // The x columns of a chunk of up to CHG steps are resident in LDS; the workgroup
   // meets only when they are replaced, and between those points every wave runs
-  // its steps at its own pace (wait for its weights, transpose them through its
-  // private tile, multiply), so that the waves of a compute unit drift apart and
-  // their memory waits, LDS traffic and arithmetic overlap.
+  // its steps at its own pace (wait for its weights, multiply), so that the
+  // waves of a compute unit drift apart and their memory waits, LDS traffic and
+  // arithmetic overlap.
   // Every wave runs the chunk loop the same number of times, whether it has
   // steps in a chunk or not: the barriers always match.  A chunk holds an even
   // number of steps of every wave, so each chunk starts on ring slot 0.
   //
   // Weight loads are issued unconditionally, also for steps past the end (those
-  // take the clamped path): a load that is issued on some paths only would force
+  // re-read the last block): a load that is issued on some paths only would force
   // the compiler to wait for *all* outstanding loads wherever it needs one of
-  // them.  For the same reason every half trip stores its ring slot to LDS,
-  // including the one past the end when the number of steps is odd.
+  // them.
   constexpr int CHG = Cfg::CHG;
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
   int s0 = 0;  // this wave's next step
@@ -492,20 +460,11 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const int s_end = min(my_steps, (c0 + CHG) / KW);
     for (; s0 < s_end; s0 += P) {
       qmm_static_for<P>([&](auto hc) {
-        constexpr int p = hc;
         const int s = s0 + hc;
         const int gs = s * KW + kw;
-        store_w(qmm_const<p>{});
-        // The loads of step s + P go out in pieces between the sub-steps of the
-        // math (the wave would otherwise sit in front of the busy address unit for
-        // the whole burst); every path issues all of them, in the same order.
-        auto issue = [&](auto tc) __attribute__((always_inline)) {
-          constexpr int t = tc;
-          load_range(qmm_const<p>{}, s + P, qmm_const<t * NLD / SUB>{}, qmm_const<(t + 1) * NLD / SUB>{});
-        };
         // (the half trip past an odd number of steps has every sub-step beyond K:
         // it issues its loads and computes nothing)
-        compute(min(gs - c0, nst - 1), s, issue);
+        compute(hc, min(gs - c0, nst - 1), s);
       });
     }
   }
@@ -677,11 +636,11 @@ int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_
   return launch_bits<XLA_AMD_DT_BF16>(a, bits, haszp, stream);
 }
 
-extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packed, const void* scale,
+extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const void* scale,
                                               const void* zp, void* out, int64_t M, int64_t N,
                                               int64_t K, int64_t C, int bits, int x_dt, int scale_dt,
                                               int zp_dt, int out_dt, void* stream) {
-  if (!x || !w_packed || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: null pointer");
+  if (!x || !w_tiled || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: null pointer");
   if (M < 0 || N <= 0 || K <= 0 || C <= 0 || K % C != 0)
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: bad sizes M=%lld N=%lld K=%lld C=%lld",
                     (long long)M, (long long)N, (long long)K, (long long)C);
@@ -695,7 +654,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packe
                     (long long)K, (long long)C);
   if (N > (1 << 30) || K > (1 << 24) || M > (1 << 30))
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: dimension too large");
-  if (((uintptr_t)x | (uintptr_t)w_packed) & 15)
+  if (((uintptr_t)x | (uintptr_t)w_tiled) & 15)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: x and w must be 16-byte aligned");
   if (((uintptr_t)out & 15) && (N & 3) == 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: out must be 16-byte aligned");
@@ -705,7 +664,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_packe
   for (int64_t m0 = 0; m0 < M; m0 += pass) {
     SkinnyArgs a;
     a.x = (const char*)x + (size_t)m0 * K * xsz;
-    a.w = (const uint8_t*)w_packed;
+    a.w = (const uint8_t*)w_tiled;
     a.scale = scale;
     a.zp = zp;
     a.out = (char*)out + (size_t)m0 * N * osz;

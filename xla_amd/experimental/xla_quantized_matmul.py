@@ -91,18 +91,13 @@ def _result_dtype(x, scaler, quantize_activation):
   return torch.promote_types(x.dtype, scaler.dtype)
 
 
-# ---- one-time K-major copies of weights ---------------------------------------
-# key id(w) -> (version, data_ptr, bits, packed tensor); dropped when w dies.
+# ---- one-time re-layouts of weights ----------------------------------------------
+# key (id(w), kind) -> (version, data_ptr, bits, copy); dropped when w dies.
 _pack_cache = {}
 
 
-def _packed_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
-  """K-major copy of w (int8 [N,K] or int4 nibbles [N,K/2]) for the streaming kernel.
-
-  The copy is made once per weight tensor and reused while the tensor is alive
-  and unmodified (same object, same storage pointer, same version counter).
-  """
-  key = id(w)
+def _relayout(w: torch.Tensor, bits: int, layout: int, kind: str) -> torch.Tensor:
+  key = (id(w), kind)
   hit = _pack_cache.get(key)
   if hit is not None and hit[0] == w._version and hit[1] == w.data_ptr() and hit[2] == bits:
     counters["pack_hit"] += 1
@@ -114,18 +109,33 @@ def _packed_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
     s, c, n = w.shape
     k = s * c
   lib = _lib.load()
-  nbytes = lib.xla_amd_qmm_packed_bytes(n, k, bits)
+  size_fn, copy_fn = ((lib.xla_amd_qmm_tiled_bytes, lib.xla_amd_qmm_tile_weight) if kind == "tiled" else
+                      (lib.xla_amd_qmm_packed_bytes, lib.xla_amd_qmm_pack_weight))
+  nbytes = size_fn(n, k, bits)
   if nbytes == 0:
-    raise RuntimeError(f"xla_amd: cannot pack weight of shape {tuple(w.shape)} to {bits} bits")
-  packed = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
-  _lib.check(
-      lib.xla_amd_qmm_pack_weight(w.data_ptr(), packed.data_ptr(), s, c, n, layout, bits,
-                                  _lib.stream_of(w)), "pack_weight")
+    raise RuntimeError(f"xla_amd: cannot re-lay out weight of shape {tuple(w.shape)} to {bits} bits ({kind})")
+  out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+  _lib.check(copy_fn(w.data_ptr(), out.data_ptr(), s, c, n, layout, bits, _lib.stream_of(w)), f"{kind} weight")
   counters["pack"] += 1
   if hit is None:
     weakref.finalize(w, _pack_cache.pop, key, None)
-  _pack_cache[key] = (w._version, w.data_ptr(), bits, packed)
-  return packed
+  _pack_cache[key] = (w._version, w.data_ptr(), bits, out)
+  return out
+
+
+def _packed_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
+  """Plain K-major copy of w (int8 [N,K] or int4 nibbles [N,K/2])."""
+  return _relayout(w, bits, layout, "packed")
+
+
+def _tiled_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
+  """Tiled copy of w for the streaming kernel (blocks of 16 channels x 128 columns in MFMA operand order).
+
+  The copy is made once per weight tensor and reused while the tensor is alive
+  and unmodified (same object, same storage pointer, same version counter); it
+  costs as much device memory again as the weight itself.
+  """
+  return _relayout(w, bits, layout, "tiled")
 
 
 def _weight_only_gpu(x2, w, scaler, zero_point, block_size, int4_weight, out_dtype):
@@ -148,7 +158,7 @@ def _weight_only_gpu(x2, w, scaler, zero_point, block_size, int4_weight, out_dty
   stream = _lib.stream_of(x2)
   zp_dt = _lib.dt(zero_point.dtype) if zero_point is not None else _lib.dt(x2.dtype)
   if kern == _lib.KERNEL_SKINNY_MFMA:
-    wk = w if (bits == 8 and not blockwise) else _packed_weight(w, bits, layout)
+    wk = _tiled_weight(w, bits, layout)
     counters["skinny_mfma"] += 1
     _lib.check(
         lib.xla_amd_qmm_weight_only_skinny(x2.data_ptr(), wk.data_ptr(), scaler.data_ptr(),
