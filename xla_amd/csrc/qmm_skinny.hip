@@ -21,8 +21,8 @@
 //
 // Synchronisation.  The workgroup meets only when the resident x columns are
 // replaced.  In between nothing is shared but read-only x, so every wave runs
-// at its own pace: wait for its weight loads (a ring of two steps in flight,
-// re-issued piecewise between the multiplies), multiply.  The waves
+// at its own pace: wait for its weight loads (one step in flight, each
+// fragment re-loaded as soon as it has been used), multiply.  The waves
 // of a compute unit drift apart, and the memory waits of one overlap the LDS
 // traffic and arithmetic of the others; a barrier per step would instead make
 // each step as slow as its slowest wave.
@@ -152,9 +152,12 @@ struct SkinnyCfg {
   static constexpr int X_TILE = XROWS * XROW;                // the x columns of one step, all rows
   static constexpr int CH = kLdsLimit / X_TILE;              // steps whose x columns are resident in LDS together
   static constexpr int XPW = X_TILE / 1024 / NW;             // 1 KB pieces of an x tile copied by each wave
-  static constexpr int P = 2;                                // steps of weight loads in flight (register ring)
-  static constexpr int CHG = CH / (2 * KW) * (2 * KW);       // ... rounded so that a chunk holds an even number of steps of every wave
-  static constexpr bool kFits = CHG >= 2 * KW;
+  // Steps of weight loads in flight per wave (register ring).  One step is
+  // 8 KB per wave, 7 MB over the chip: enough to cover the memory latency; with
+  // two or more the measured time goes *up* (the extra requests only queue).
+  static constexpr int P = 1;
+  static constexpr int CHG = CH / (P * KW) * (P * KW);       // ... rounded so that a chunk holds whole trips around the ring for every wave
+  static constexpr bool kFits = CHG >= P * KW;
   static constexpr int kRedBytes = NW * 16 * MT * 256;       // cross-wave reduction scratch (reuses the x tiles)
   static constexpr int lds_bytes(int steps) {
     const int x = (steps < CHG ? steps : CHG) * X_TILE;
@@ -441,29 +444,39 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // waves of a compute unit drift apart and their memory waits, LDS traffic and
   // arithmetic overlap.
   // Every wave runs the chunk loop the same number of times, whether it has
-  // steps in a chunk or not: the barriers always match.  A chunk holds an even
-  // number of steps of every wave, so each chunk starts on ring slot 0.
+  // steps in a chunk or not: the barriers always match.  A chunk holds whole
+  // trips around the ring for every wave, so each chunk starts on ring slot 0.
   //
   // Weight loads are issued unconditionally, also for steps past the end (those
   // re-read the last block): a load that is issued on some paths only would force
   // the compiler to wait for *all* outstanding loads wherever it needs one of
   // them.
   constexpr int CHG = Cfg::CHG;
+  // First chunk: the x copies go out first and the weight ring after them, so
+  // that waiting for x (loads complete in order) leaves the weight loads in flight.
+  x_chunk_load(0, min(CHG, steps_total));
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
+  {
+    constexpr int kInFlight = P * NLD;  // vmcnt(kInFlight): everything older than the ring has landed
+    __builtin_amdgcn_s_waitcnt(((kInFlight >> 4) << 14) | 0x0F70 | (kInFlight & 15));
+  }
+  qmm_lds_barrier();
   int s0 = 0;  // this wave's next step
   for (int c0 = 0; c0 < steps_total; c0 += CHG) {
     const int nst = min(CHG, steps_total - c0);
-    if (c0 > 0) qmm_lds_barrier();       // every wave has finished reading the old columns
-    x_chunk_load(c0, nst);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
-    qmm_lds_barrier();
+    if (c0 > 0) {
+      qmm_lds_barrier();                   // every wave has finished reading the old columns
+      x_chunk_load(c0, nst);
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+      qmm_lds_barrier();
+    }
     const int s_end = min(my_steps, (c0 + CHG) / KW);
     for (; s0 < s_end; s0 += P) {
       qmm_static_for<P>([&](auto hc) {
         const int s = s0 + hc;
         const int gs = s * KW + kw;
-        // (the half trip past an odd number of steps has every sub-step beyond K:
-        // it issues its loads and computes nothing)
+        // (a step past the end, which only occurs to complete a trip around the
+        // ring, has every sub-step beyond K: it issues its loads and computes nothing)
         compute(hc, min(gs - c0, nst - 1), s);
       });
     }
@@ -592,13 +605,6 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
     if (a.N < 200 * 32 && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
   }
   if (kw == 1) {
-    // Large N, per-channel int8, up to 16 rows: 8 waves per workgroup (two per
-    // SIMD, so that one wave's waits are another's issue slots) as 4 row groups
-    // x 2 k-splits, walking K in steps of 256 columns.
-    if constexpr (BITS == 8 && MT == 1 && XT != XLA_AMD_DT_F32) {
-      if (perch) return haszp ? launch_kernel<XT, 8, 1, 2, kRedRaw, true, 8, 256>(a, stream)
-                              : launch_kernel<XT, 8, 1, 2, kRedRaw, false, 8, 256>(a, stream);
-    }
     return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
                  : launch_zp<XT, BITS, MT, 1, kRedNone>(a, haszp, stream);
   }
