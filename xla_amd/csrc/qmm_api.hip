@@ -51,7 +51,8 @@ extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, 
     return XLA_AMD_KERNEL_W8A8_GENERIC;
   }
   if (C <= 0) C = K;
-  if (K % 128 == 0 && C % 128 == 0 && (bits == 8 || bits == 4) && M >= 1)
+  if (K % 128 == 0 && C % 128 == 0 && (bits == 8 || bits == 4) && M >= 1 &&
+      (C == K || (N % 4 == 0 && (K / C) * N >= 8)))  // blockwise: vector loads of 4 channels' scales
     return XLA_AMD_KERNEL_SKINNY_MFMA;
   return XLA_AMD_KERNEL_GENERIC;
 }

@@ -300,7 +300,41 @@ qmm_skinny_kernel(SkinnyArgs a) {
       if constexpr (HASZP) pre_zp[v] = qmm_load_raw(a.zp, n, a.zp_dt);
     });
   }
-  auto block_epilogue = [&](int sblk) __attribute__((always_inline)) {
+  // Blockwise: scale / zero point of 4 consecutive channels are one 16-byte
+  // load (8 of them used for 2-byte types), fetched one step ahead: bw_sc[t]
+  // holds those of the block that sub-step t of the current step lies in.
+  // (The entry point admits blockwise problems only with N % 4 == 0, for the
+  // alignment, and at least 16 bytes of scales.)
+  constexpr int kBw = RED == kRedRaw ? 1 : SUB;
+  i32x4 bw_sc[kBw], bw_zp[kBw];
+  int bw_sc_sel[kBw], bw_zp_sel[kBw];  // 2-byte types: 0 or 2, the dword pair of the load that holds the values
+  const int n_sblk = K / C;
+  auto bw_fetch1 = [&](const void* base, int dt, int sblk, i32x4& dst, int& sel) __attribute__((always_inline)) {
+    const int esz = dt == XLA_AMD_DT_F32 ? 4 : 2;
+    const int64_t total = (int64_t)n_sblk * N * esz;
+    const int64_t off = ((int64_t)sblk * N + min(n_wave + 4 * g, N - 4)) * esz;
+    const int64_t at = min(off, total - 16);  // a 2-byte row end: read the 16 bytes that end there
+    sel = (int)(off - at) >> 2;
+    dst = *(const i32x4*)((const char*)base + at);
+  };
+  // scales of the block that sub-step t of this wave's s-th step lies in
+  auto bw_fetch = [&](int s, auto tc) __attribute__((always_inline)) {
+    constexpr int t = tc;
+    if constexpr (RED != kRedRaw) {
+      const int sblk = min(((s * KW + kw) * KS + t * 128) / C, n_sblk - 1);
+      bw_fetch1(a.scale, a.scale_dt, sblk, bw_sc[t], bw_sc_sel[t]);
+      if constexpr (HASZP) bw_fetch1(a.zp, a.zp_dt, sblk, bw_zp[t], bw_zp_sel[t]);
+    }
+  };
+  auto bw_value = [&](const i32x4& raw, int sel, int dt, auto vc) __attribute__((always_inline)) -> float {
+    constexpr int v = vc;
+    if (dt == XLA_AMD_DT_F32) return __int_as_float(raw[v]);
+    const uint32_t lo = (uint32_t)(sel ? raw[2] : raw[0]), hi = (uint32_t)(sel ? raw[3] : raw[1]);
+    const uint32_t dw = (v >> 1) ? hi : lo;
+    return qmm_from_raw((v & 1) ? (dw >> 16) : (dw & 0xffffu), dt);
+  };
+  auto block_epilogue = [&](int sblk, auto tc) __attribute__((always_inline)) {
+    constexpr int t = tc;
     qmm_static_for<4>([&](auto vc) {
       constexpr int v = vc;
       const int n = min(n_wave + 4 * g + v, N - 1);
@@ -309,8 +343,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
         sc = qmm_from_raw(pre_sc[v], a.scale_dt);
         if constexpr (HASZP) zv = qmm_from_raw(pre_zp[v], a.zp_dt);
       } else {
-        sc = qmm_load(a.scale, (int64_t)sblk * N + n, a.scale_dt);
-        if constexpr (HASZP) zv = qmm_load(a.zp, (int64_t)sblk * N + n, a.zp_dt);
+        sc = bw_value(bw_sc[t], bw_sc_sel[t], a.scale_dt, vc);
+        if constexpr (HASZP) zv = bw_value(bw_zp[t], bw_zp_sel[t], a.zp_dt, vc);
       }
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
@@ -402,7 +436,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
       }
       if constexpr (RED != kRedRaw) {
         if (--block_left == 0) {
-          block_epilogue(k_sub / C);
+          block_epilogue(k_sub / C, tc);
           block_left = sub_per_block;
         }
       }
@@ -422,6 +456,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         if (k_step + t * 128 < K) math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq[cur]);
         load_sub(pc, s + P, tc);
+        bw_fetch(s + 1, tc);
         __builtin_amdgcn_sched_barrier(0);
       });
     } else {
@@ -433,6 +468,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
           math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq);
         }
         load_sub(pc, s + P, tc);
+        bw_fetch(s + 1, tc);
       });
     }
   };
@@ -456,8 +492,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // that waiting for x (loads complete in order) leaves the weight loads in flight.
   x_chunk_load(0, min(CHG, steps_total));
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
+  qmm_static_for<kBw>([&](auto tc) { bw_fetch(0, tc); });
   {
-    constexpr int kInFlight = P * NLD;  // vmcnt(kInFlight): everything older than the ring has landed
+    // vmcnt(kInFlight): everything older than the ring and the first scales has landed
+    constexpr int kInFlight = P * NLD + (RED != kRedRaw ? (HASZP ? 2 : 1) * kBw : 0);
     __builtin_amdgcn_s_waitcnt(((kInFlight >> 4) << 14) | 0x0F70 | (kInFlight & 15));
   }
   qmm_lds_barrier();
@@ -526,7 +564,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
       }
     });
   }
-  if constexpr (RED == kRedRaw) block_epilogue(0);  // the single block ends here
+  if constexpr (RED == kRedRaw) block_epilogue(0, qmm_const<0>{});  // the single block ends here
 
   qmm_static_for<MT>([&](auto mc) {
     constexpr int mt = mc;
@@ -658,6 +696,9 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
   if (K % 128 != 0 || C % 128 != 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: K=%lld and C=%lld must be multiples of 128",
                     (long long)K, (long long)C);
+  if (C != K && (N % 4 != 0 || (K / C) * N < 8))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: blockwise needs N %% 4 == 0 and >= 8 scales (N=%lld)",
+                    (long long)N);
   if (N > (1 << 30) || K > (1 << 24) || M > (1 << 30))
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: dimension too large");
   if (((uintptr_t)x | (uintptr_t)w_tiled) & 15)
