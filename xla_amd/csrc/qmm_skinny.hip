@@ -372,8 +372,12 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // out between the multiplies instead of as one burst.  Sub-steps at or beyond K
   // are skipped (a uniform branch around arithmetic only: the loads stay in
   // straight-line code, so the compiler's wait counts for the ring stay exact).
-  auto compute = [&](auto pc, int tile, int s) __attribute__((always_inline)) {
+  // refill = 0 is the wave's last step: nothing is fetched for later steps, so
+  // that the epilogue does not have to wait for loads nobody reads before it may
+  // reuse their registers.
+  auto compute = [&](auto pc, int tile, int s, auto refillc) __attribute__((always_inline)) {
     constexpr int p = pc;
+    constexpr bool kRefill = refillc != 0;
     const char* xb = smem + tile * X_TILE;
     const int k_step = (s * KW + kw) * KS;
     if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
@@ -455,8 +459,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
         if constexpr (t + 1 < SUB) read_frags(qmm_const<t + 1>{}, xq[nxt]);
         __builtin_amdgcn_sched_barrier(0);
         if (k_step + t * 128 < K) math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq[cur]);
-        load_sub(pc, s + P, tc);
-        bw_fetch(s + 1, tc);
+        if constexpr (kRefill) {
+          load_sub(pc, s + P, tc);
+          bw_fetch(s + 1, tc);
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
     } else {
@@ -467,8 +473,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
           read_frags(tc, xq);
           math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq);
         }
-        load_sub(pc, s + P, tc);
-        bw_fetch(s + 1, tc);
+        if constexpr (kRefill) {
+          load_sub(pc, s + P, tc);
+          bw_fetch(s + 1, tc);
+        }
       });
     }
   };
@@ -488,14 +496,15 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // the compiler to wait for *all* outstanding loads wherever it needs one of
   // them.
   constexpr int CHG = Cfg::CHG;
-  // First chunk: the x copies go out first and the weight ring after them, so
-  // that waiting for x (loads complete in order) leaves the weight loads in flight.
-  x_chunk_load(0, min(CHG, steps_total));
+  // First chunk: the first step's weights (the longest latency) go out first,
+  // then the x copies, then the first scales; loads complete in order, so waiting
+  // for the x copies also waits for those weights, which step 0 needs anyway.
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
+  x_chunk_load(0, min(CHG, steps_total));
   qmm_static_for<kBw>([&](auto tc) { bw_fetch(0, tc); });
   {
-    // vmcnt(kInFlight): everything older than the ring and the first scales has landed
-    constexpr int kInFlight = P * NLD + (RED != kRedRaw ? (HASZP ? 2 : 1) * kBw : 0);
+    // vmcnt(kInFlight): everything older than the first scales has landed
+    constexpr int kInFlight = RED != kRedRaw ? (HASZP ? 2 : 1) * kBw : 0;
     __builtin_amdgcn_s_waitcnt(((kInFlight >> 4) << 14) | 0x0F70 | (kInFlight & 15));
   }
   qmm_lds_barrier();
@@ -508,15 +517,23 @@ qmm_skinny_kernel(SkinnyArgs a) {
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
       qmm_lds_barrier();
     }
-    const int s_end = min(my_steps, (c0 + CHG) / KW);
+    int s_end = min(my_steps, (c0 + CHG) / KW);
+    // Without k-splits the wave's last step lies in the last chunk: it is run
+    // after the loop, in a form that fetches nothing more.
+    if constexpr (KW == 1 && P == 1) {
+      if (c0 + CHG >= steps_total) --s_end;
+    }
     for (; s0 < s_end; s0 += P) {
       qmm_static_for<P>([&](auto hc) {
         const int s = s0 + hc;
         const int gs = s * KW + kw;
         // (a step past the end, which only occurs to complete a trip around the
         // ring, has every sub-step beyond K: it issues its loads and computes nothing)
-        compute(hc, min(gs - c0, nst - 1), s);
+        compute(hc, min(gs - c0, nst - 1), s, qmm_const<1>{});
       });
+    }
+    if constexpr (KW == 1 && P == 1) {
+      if (c0 + CHG >= steps_total) compute(qmm_const<0>{}, s0 - c0, s0, qmm_const<0>{});
     }
   }
 
