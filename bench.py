@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA (5.0 POP/s)
 
 N_OUT, K_IN = 14336, 4096
-TRAFFIC_BYTES_PER_LAUNCH = 68.9e6  # decode GEMV M=16, see profiles/skinny_gemv_cfg2_m16_hbm_traffic.md
+TRAFFIC_BYTES_PER_LAUNCH = 60.4e6  # decode GEMV M=16, see profiles/skinny_gemv_cfg2_m16_hbm_traffic.md
 
 
 def gemv_bytes(m, n, k, w_bytes_per_elem=1.0, x_b=2, s_b=2, out_b=2, n_scale_rows=1, zp=False):
