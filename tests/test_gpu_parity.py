@@ -339,6 +339,26 @@ def test_w8a8_tiles_and_tails(ops):
       assert torch.equal(acc.cpu().long(), ref), (bm, m, n, k)
 
 
+def test_w8a8_column_split_two_tile_widths(ops):
+  # a shape whose 256-wide tiles would leave the last round of workgroups mostly empty: the library covers the
+  # columns with 256-wide and 192-wide tiles in two launches; ragged last tile, partial last K step
+  m, n, k = 2048, 14436, 192
+  g = cases.gen(99)
+  xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+  w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+  xs, ws = torch.rand(m, 1, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
+  ref = torch.from_numpy(xq.numpy().astype(np.int64) @ w.numpy().astype(np.int64).T)
+  out, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), xs.cuda(), ws.cuda(), None, None, cvt_dtype=torch.float32,
+                               mid_dtype=torch.float32, out_dtype=torch.float32, want_acc=True)
+  assert torch.equal(acc.cpu().long(), ref)
+  expect = (ref.float() * ws[None, :]) * xs
+  assert torch.equal(out.cpu(), expect)
+  # short epilogue (no accumulator output), bf16
+  out16, _ = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), xs.cuda(), ws.cuda(), None, None, cvt_dtype=torch.float32,
+                               mid_dtype=torch.float32, out_dtype=torch.bfloat16)
+  assert torch.equal(out16.cpu(), expect.to(torch.bfloat16))
+
+
 def test_skinny_k_splits_and_long_k(ops):
   # small N takes k-split workgroups; K = 14336 is the down projection; M > 32 takes two passes
   for (m, n, k, xdt) in [(16, 256, 4096, torch.bfloat16), (5, 4096, 14336, torch.bfloat16), (40, 1024, 1024, torch.bfloat16),

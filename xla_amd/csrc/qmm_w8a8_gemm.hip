@@ -37,6 +37,7 @@ struct GemmArgs {
   void* out;
   int32_t* acc_out;
   int M, N, K;
+  int ldo;  // elements between rows of out / acc_out (N, or more when this launch covers a column range)
   int x_scale_dt, w_scale_dt, zp_dt, cvt_dt, mid_dt, zpo_dt, out_dt;
   int tiles_m, tiles_n;
 };
@@ -249,9 +250,11 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
     if (m0 + BM <= g.M && n0 + BN <= g.N) {
       // Whole tile, f32 chain: out = cast((float(acc) * w_scale) * x_scale).  The lane's
       // 4 columns are the same in every pass, so their scales stay in registers.
-      const int c4 = lane % kLanesPerRow, prow = lane / kLanesPerRow;
-      const f32x4 ws = *(const f32x4*)(s_ws + wn * TN + c4 * 4);
-      const int n = n0 + wn * TN + c4 * 4;
+      // (when the lanes of a row divide the wave, a lane's 4 columns are the same
+      // in every pass and their scales stay in registers)
+      constexpr bool kFixedCols = 64 % kLanesPerRow == 0;
+      const int c4f = lane % kLanesPerRow, prow = lane / kLanesPerRow;
+      const f32x4 wsf = *(const f32x4*)(s_ws + wn * TN + c4f * 4);
       qmm_static_for<MI>([&](auto ic) {
         constexpr int i = ic;
         qmm_static_for<NI>([&](auto jc) {
@@ -261,15 +264,23 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
             s_ep[(8 * (v >> 2) + 4 * lchunk + (v & 3)) * kEpStride + j * 32 + lrow] = acc[i][j][v];
           });
         });
-        const int rbase = wm * TM + i * 32 + prow;
+        const int rbase = wm * TM + i * 32;
 #pragma unroll 4
         for (int p = 0; p < kPasses; ++p) {
-          const int row = p * kRowsPerPass;
-          const i32x4 a = *(const i32x4*)(s_ep + (row + prow) * kEpStride + c4 * 4);
+          int row, c4;
+          f32x4 ws;
+          if constexpr (kFixedCols) {
+            row = p * kRowsPerPass + prow; c4 = c4f; ws = wsf;
+          } else {
+            const int idx = p * 64 + lane;
+            row = idx / kLanesPerRow; c4 = idx % kLanesPerRow;
+            ws = *(const f32x4*)(s_ws + wn * TN + c4 * 4);
+          }
+          const i32x4 a = *(const i32x4*)(s_ep + row * kEpStride + c4 * 4);
           const float xs = s_xs[rbase + row];
           const float v0 = ((float)a[0] * ws[0]) * xs, v1 = ((float)a[1] * ws[1]) * xs;
           const float v2 = ((float)a[2] * ws[2]) * xs, v3 = ((float)a[3] * ws[3]) * xs;
-          const size_t idx0 = (size_t)(m0 + rbase + row) * g.N + n;
+          const size_t idx0 = (size_t)(m0 + rbase + row) * g.ldo + (n0 + wn * TN + c4 * 4);
           if constexpr (EPI == 3) {
             *(f32x4*)((float*)g.out + idx0) = f32x4{v0, v1, v2, v3};
           } else if constexpr (EPI == 1) {
@@ -287,7 +298,7 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
     }
   }
   const bool simple = g.cvt_dt == XLA_AMD_DT_F32 && g.mid_dt == XLA_AMD_DT_F32 && !has_zp;
-  const bool n_vec = (g.N % 4) == 0;  // rows of out start 8/16-byte aligned
+  const bool n_vec = (g.ldo % 4) == 0 && (g.N % 4) == 0;  // rows of out start 8/16-byte aligned, no ragged last group
   // Finishes one staged 32 x TN block whose first row is global row mb.
   auto finish_block = [&](int mb, int row_off) {
     for (int p = 0; p < kPasses; ++p) {
@@ -296,7 +307,7 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
       const int m = mb + row, n = n0 + wn * TN + c4 * 4;
       if (m >= g.M || n >= g.N) continue;
       const i32x4 a = *(const i32x4*)(s_ep + row * kEpStride + c4 * 4);
-      const size_t idx0 = (size_t)m * g.N + n;
+      const size_t idx0 = (size_t)m * g.ldo + n;
       const int nvalid = min(4, g.N - n);
       if (want_acc) {
         if (n_vec) *(i32x4*)(g.acc_out + idx0) = a;
@@ -376,7 +387,7 @@ int launch_tile_epi(GemmArgs g, hipStream_t stream) {
 template <int BM, int BN, int WM, int WN>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const bool fast = g.out && !g.acc_out && !g.zp && g.cvt_dt == XLA_AMD_DT_F32 &&
-                    g.mid_dt == XLA_AMD_DT_F32 && (g.N % 4) == 0 && (((uintptr_t)g.out) & 15) == 0;
+                    g.mid_dt == XLA_AMD_DT_F32 && (g.N % 4) == 0 && (g.ldo % 4) == 0 && (((uintptr_t)g.out) & 15) == 0;
   if (fast && g.out_dt == XLA_AMD_DT_BF16) return launch_tile_epi<BM, BN, WM, WN, 1>(g, stream);
   if (fast && g.out_dt == XLA_AMD_DT_F16) return launch_tile_epi<BM, BN, WM, WN, 2>(g, stream);
   if (fast && g.out_dt == XLA_AMD_DT_F32) return launch_tile_epi<BM, BN, WM, WN, 3>(g, stream);
@@ -429,7 +440,7 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
   GemmArgs g;
   g.a = x_q; g.b = w; g.x_scale = x_scale; g.w_scale = w_scale; g.zp = out ? zp : nullptr;
   g.x_sum = x_sum; g.out = out; g.acc_out = acc_out;
-  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K; g.ldo = (int)N;
   g.x_scale_dt = x_scale_dt; g.w_scale_dt = w_scale_dt; g.zp_dt = zp_dt; g.cvt_dt = cvt_dt;
   g.mid_dt = mid_dt; g.zpo_dt = zpo_dt; g.out_dt = out_dt;
   g.tiles_m = g.tiles_n = 0;
@@ -437,7 +448,44 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
   if (bm == 0 && bn == 0) choose_tile(M, N, &bm, &bn);
   // 256x256: 8 waves (2 x 4, wave tile 128 x 64): two waves per SIMD, so that one wave's LDS and
   // barrier waits are the other's MFMA slots (measured 128 us against 154 us with 4 waves of 128 x 128)
-  if (bm == 256 && bn == 256) return launch_tile<256, 256, 2, 4>(g, s);
+  if (bm == 256 && bn == 256) {
+    // Rounds of tiles over the 256 CUs: a last round that is only partly full costs a
+    // whole round.  Columns can be covered by n1 tiles of 256 followed by n2 tiles of
+    // 192 (two launches); pick the split with the least estimated time (a round of
+    // 256 x 192 tiles takes 3/4 of a round of 256 x 256 tiles).  cfg4 (2048 x 14336):
+    // 8 x 56 = 448 tiles = 2 rounds becomes 8 x 32 + 8 x 32 = 1 + 0.75 rounds.
+    int64_t best_n1 = (N + 255) / 256;
+    if (block_m == 0 && block_n == 0) {
+      const int64_t mt = (M + 255) / 256;
+      auto rounds = [](int64_t tiles) { return (double)((tiles + 255) / 256); };
+      double best = rounds(mt * best_n1);
+      for (int64_t n1 = N / 256; n1 >= 0; --n1) {
+        const int64_t n2 = (N - n1 * 256 + 191) / 192;
+        if (n2 <= 0) continue;
+        const double cost = rounds(mt * n1) + 0.75 * rounds(mt * n2) + (n1 > 0 ? 0.02 : 0.0);
+        if (cost < best - 1e-9) { best = cost; best_n1 = n1; }
+      }
+    }
+    const int64_t N1 = best_n1 * 256 < N ? best_n1 * 256 : N;
+    int rc = XLA_AMD_QMM_OK;
+    if (N1 > 0) {
+      GemmArgs g1 = g;
+      g1.N = (int)N1;
+      rc = launch_tile<256, 256, 2, 4>(g1, s);
+      if (rc != XLA_AMD_QMM_OK) return rc;
+    }
+    if (N1 < N) {
+      GemmArgs g2 = g;
+      g2.N = (int)(N - N1);
+      g2.b = w + (size_t)N1 * K;
+      if (g.w_scale) g2.w_scale = (const char*)g.w_scale + (size_t)N1 * qmm_dt_size(w_scale_dt);
+      if (g.zp) g2.zp = (const char*)g.zp + (size_t)N1 * qmm_dt_size(zp_dt);
+      if (g.out) g2.out = (char*)g.out + (size_t)N1 * qmm_dt_size(out_dt);
+      if (g.acc_out) g2.acc_out = g.acc_out + N1;
+      rc = launch_tile<256, 192, 4, 2>(g2, s);
+    }
+    return rc;
+  }
   if (bm == 128 && bn == 128) return launch_tile<128, 128, 2, 2>(g, s);
   if (bm == 64 && bn == 64) return launch_tile<64, 64, 2, 2>(g, s);
   return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_gemm: no kernel for tile %dx%d", bm, bn);
