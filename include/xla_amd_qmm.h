@@ -121,7 +121,9 @@ int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, 
  *   zero point:            out -= rowsum/blocksum(x) (x) zp    (:125-133)
  * x [M,K] (bf16/f16/f32), w_tiled from xla_amd_qmm_tile_weight, scale [S,N],
  * zp [S,N] or NULL, out [M,N].
- * Needs K % 128 == 0 and C % 128 == 0; else XLA_AMD_QMM_EUNSUPPORTED.
+ * Needs K % 128 == 0 and C % 128 == 0; blockwise (C < K) also needs N % 4 == 0
+ * and scale / zp of x's dtype (the reference's einsum raises on mixed dtypes);
+ * else XLA_AMD_QMM_EUNSUPPORTED.
  * out_dt must be the torch promotion of (x_dt, scale_dt).
  */
 int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const void* scale,

@@ -304,11 +304,14 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // load (8 of them used for 2-byte types), fetched one step ahead: bw_sc[t]
   // holds those of the block that sub-step t of the current step lies in.
   // (The entry point admits blockwise problems only with N % 4 == 0, for the
-  // alignment, and at least 16 bytes of scales.)
+  // alignment, at least 16 bytes of scales, and scales / zero points of x's
+  // dtype, as the reference's einsum requires: the conversions below are then
+  // free of run-time dtype branches.)
   constexpr int kBw = RED == kRedRaw ? 1 : SUB;
   i32x4 bw_sc[kBw], bw_zp[kBw];
   int bw_sc_sel[kBw], bw_zp_sel[kBw];  // 2-byte types: 0 or 2, the dword pair of the load that holds the values
   const int n_sblk = K / C;
+  const int c_shift = (C & (C - 1)) == 0 ? __builtin_ctz(C) : -1;  // block size a power of two: shift instead of divide
   auto bw_fetch1 = [&](const void* base, int dt, int sblk, i32x4& dst, int& sel) __attribute__((always_inline)) {
     const int esz = dt == XLA_AMD_DT_F32 ? 4 : 2;
     const int64_t total = (int64_t)n_sblk * N * esz;
@@ -321,9 +324,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
   auto bw_fetch = [&](int s, auto tc) __attribute__((always_inline)) {
     constexpr int t = tc;
     if constexpr (RED != kRedRaw) {
-      const int sblk = min(((s * KW + kw) * KS + t * 128) / C, n_sblk - 1);
-      bw_fetch1(a.scale, a.scale_dt, sblk, bw_sc[t], bw_sc_sel[t]);
-      if constexpr (HASZP) bw_fetch1(a.zp, a.zp_dt, sblk, bw_zp[t], bw_zp_sel[t]);
+      const int k_at = (s * KW + kw) * KS + t * 128;
+      const int sblk = min(c_shift >= 0 ? (k_at >> c_shift) : k_at / C, n_sblk - 1);
+      bw_fetch1(a.scale, XT, sblk, bw_sc[t], bw_sc_sel[t]);
+      if constexpr (HASZP) bw_fetch1(a.zp, XT, sblk, bw_zp[t], bw_zp_sel[t]);
     }
   };
   auto bw_value = [&](const i32x4& raw, int sel, int dt, auto vc) __attribute__((always_inline)) -> float {
@@ -343,8 +347,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
         sc = qmm_from_raw(pre_sc[v], a.scale_dt);
         if constexpr (HASZP) zv = qmm_from_raw(pre_zp[v], a.zp_dt);
       } else {
-        sc = bw_value(bw_sc[t], bw_sc_sel[t], a.scale_dt, vc);
-        if constexpr (HASZP) zv = bw_value(bw_zp[t], bw_zp_sel[t], a.zp_dt, vc);
+        sc = bw_value(bw_sc[t], bw_sc_sel[t], XT, vc);
+        if constexpr (HASZP) zv = bw_value(bw_zp[t], bw_zp_sel[t], XT, vc);
       }
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
@@ -713,8 +717,9 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
   if (K % 128 != 0 || C % 128 != 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: K=%lld and C=%lld must be multiples of 128",
                     (long long)K, (long long)C);
-  if (C != K && (N % 4 != 0 || (K / C) * N < 8))
-    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: blockwise needs N %% 4 == 0 and >= 8 scales (N=%lld)",
+  if (C != K && (N % 4 != 0 || (K / C) * N < 8 || scale_dt != x_dt || (zp && zp_dt != x_dt)))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED,
+                    "weight_only_skinny: blockwise needs N %% 4 == 0, >= 8 scales and scale / zero point of x's dtype (N=%lld)",
                     (long long)N);
   if (N > (1 << 30) || K > (1 << 24) || M > (1 << 30))
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: dimension too large");
