@@ -209,6 +209,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
   uint32_t x_off[XPW];  // per lane: byte offset of its source chunk from the step's first column of row 0
   int x_col[XPW];       // per lane: byte column of that chunk within the step
   int x_lds[XPW];       // uniform: LDS offset of the piece within a tile
+  bool x_used[XPW];     // uniform: the piece holds at least one row below M (rows from M on are never
+                        // stored, so their x is not copied: a decode step of one row copies 1/16 of the tile)
   qmm_static_for<XPW>([&](auto jc) {
     constexpr int j = jc;
     const int q = wave * XPW + j;
@@ -218,6 +220,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
     x_col[j] = ((piece * 64 + lane % kLanesPerRow) ^ (row & 15)) * 16;
     x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + x_col[j];
     x_lds[j] = row0 * XROW + piece * 1024;
+    x_used[j] = row0 < M;
   });
 
   const int steps_total = (K + KS - 1) / KS;
@@ -252,7 +255,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
       if ((gs + 1) * KS <= K) {
         qmm_static_for<XPW>([&](auto jc) {
           constexpr int j = jc;
-          __builtin_amdgcn_global_load_lds((const void*)(xp + x_off[j]), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
+          if (x_used[j]) __builtin_amdgcn_global_load_lds((const void*)(xp + x_off[j]), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
         });
       } else {
         // last, partial step: chunks past K re-read the last valid 16 bytes of the row
@@ -261,7 +264,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
           constexpr int j = jc;
           // x_left >= 256 here, so 0 <= back <= x_col[j] <= x_off[j]
           const int back = max(x_col[j] + 16 - x_left, 0);
-          __builtin_amdgcn_global_load_lds((const void*)(xp + ((int64_t)x_off[j] - back)), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
+          if (x_used[j]) __builtin_amdgcn_global_load_lds((const void*)(xp + ((int64_t)x_off[j] - back)), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
         });
       }
     }
