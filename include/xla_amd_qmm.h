@@ -47,6 +47,12 @@ extern "C" {
 /* float -> int8 conversion of a rounded value outside [-128,127]
  * (reference: `.to(torch.int8)` with no clamp, xla_quantized_matmul.py:72;
  * XLA's ConvertElementType saturates, torch's CPU cast wraps modulo 256). */
+/* integer dtypes of quantized tensors (quantize_affine / dequantize_affine) */
+#define XLA_AMD_QDT_I8 0
+#define XLA_AMD_QDT_U8 1
+#define XLA_AMD_QDT_I16 2
+#define XLA_AMD_QDT_I32 3
+
 #define XLA_AMD_OVERFLOW_SATURATE 0
 #define XLA_AMD_OVERFLOW_WRAP 1
 
@@ -202,6 +208,33 @@ int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, int bits, i
  * get_tuned_block_sizes (pallas_kernels/quantized_matmul_kernel.py:537-555).
  */
 int xla_amd_qmm_w8a8_tile(int64_t M, int64_t N, int64_t K, int32_t* tile_mnk /* host */);
+
+/*
+ * Affine quantization of a whole tensor, per tensor (channels == 1) or per
+ * channel; the contiguous tensor is read as [outer, channels, inner].
+ *   q[o,c,i] = cast(clamp(rint(f32(x[o,c,i]) * inv_scale[c]) + zp[c], qmin, qmax))
+ * (all in f32, rint = half to even, NaN -> 0): the decomposition that
+ * quantized_decomposed::quantize_per_tensor / quantize_per_channel denote
+ * (bound to XLA in torch_xla/experimental/quantized.py:7-22, where they lower
+ * to stablehlo.uniform_quantize through _xla_quantize_tensor,
+ * csrc/init_python_bindings.cpp:1964).  inv_scale and zp are device arrays of
+ * `channels` entries.
+ */
+int xla_amd_qmm_quantize_affine(const void* x, void* q, const float* inv_scale, const int32_t* zp,
+                                int64_t outer, int64_t channels, int64_t inner, int x_dt, int q_dt,
+                                int32_t qmin, int32_t qmax, void* stream);
+
+/*
+ * Affine dequantization (quantized_decomposed::dequantize_per_tensor /
+ * dequantize_per_channel, torch_xla/experimental/quantized.py:25-41).
+ *   int_subtract != 0: out = cast(f32(q - zp[c]) * scale[c])            (per-channel form)
+ *   int_subtract == 0: out = round(round(cast(q) - zp[c]) * scale[c]),  each result rounded to out's dtype,
+ *                      zp and scale entering as f32 scalars            (per-tensor form)
+ * zp may be NULL (zero).
+ */
+int xla_amd_qmm_dequantize_affine(const void* q, void* out, const float* scale, const int32_t* zp,
+                                  int64_t outer, int64_t channels, int64_t inner, int q_dt, int out_dt,
+                                  int int_subtract, void* stream);
 
 #ifdef __cplusplus
 }

@@ -390,3 +390,46 @@ def test_module_and_state_dict_on_gpu(ops):
     assert out.shape == (3, 7, 64)
     check(out, exp, f"module {kw}")
     assert qd.weight.is_cuda and set(qd.state_dict()) >= {"weight", "weight_scaler"}
+
+
+# ---- quantized_decomposed quantize / dequantize on the GPU ------------------------------------------
+
+def test_qdq_ops_match_oracle_and_torch_cpu(ops):
+  import xla_amd.experimental.quantized  # noqa: F401  (binds the CUDA key)
+  from oracle import quantized_decomposed_oracle as qo
+  qd = torch.ops.quantized_decomposed
+  g = torch.Generator().manual_seed(5)
+  x = torch.randn(6, 10, 16, generator=g) * 3
+  x[0, 0, :8] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 1e9, -1e9, 0.0])
+  for xdt in (torch.float32, torch.bfloat16, torch.float16):
+    xi = x.to(xdt)
+    for (scale, zp, lo, hi, dt, ndt) in [(0.037, -5, -128, 127, torch.int8, np.int8), (0.11, 128, 0, 255, torch.uint8, np.uint8),
+                                         (0.01, 10, -32768, 32767, torch.int16, np.int16)]:
+      q = qd.quantize_per_tensor(xi.cuda(), scale, zp, lo, hi, dt)
+      assert q.dtype == dt and q.is_cuda
+      expect = qo.quantize_affine(xi.float().numpy(), np.float32(1.0 / scale), zp, lo, hi, ndt)
+      assert np.array_equal(q.cpu().numpy(), expect), (xdt, scale)
+      assert torch.equal(q.cpu(), qd.quantize_per_tensor(xi, scale, zp, lo, hi, dt))
+      d = qd.dequantize_per_tensor(q, scale, zp, lo, hi, dt)
+      assert np.array_equal(d.cpu().numpy(), qo.dequantize_per_tensor_f32(expect, scale, zp))
+      d16 = qd.dequantize_per_tensor(q, scale, zp, lo, hi, dt, out_dtype=torch.bfloat16)
+      assert torch.equal(d16.cpu(), qd.dequantize_per_tensor(q.cpu(), scale, zp, lo, hi, dt, out_dtype=torch.bfloat16))
+    for axis in (0, 1, 2):
+      c = x.shape[axis]
+      g2 = torch.Generator().manual_seed(axis)
+      scales = torch.rand(c, generator=g2) * 0.1 + 0.01
+      zps = torch.randint(-20, 20, (c,), generator=g2)
+      q = qd.quantize_per_channel(xi.cuda(), scales.cuda(), zps.cuda(), axis, -128, 127, torch.int8)
+      expect = qo.quantize_affine(xi.float().numpy(), (1.0 / scales).numpy(), zps.numpy(), -128, 127, np.int8, axis)
+      assert np.array_equal(q.cpu().numpy(), expect), (xdt, axis)
+      d = qd.dequantize_per_channel(q, scales.cuda(), zps.cuda(), axis, -128, 127, torch.int8)
+      assert np.array_equal(d.cpu().numpy(), qo.dequantize_per_channel(expect, scales.numpy(), zps.numpy(), axis))
+      d0 = qd.dequantize_per_channel(q, scales.cuda(), None, axis, -128, 127, torch.int8)
+      assert np.array_equal(d0.cpu().numpy(), qo.dequantize_per_channel(expect, scales.numpy(), None, axis))
+  # a weight-sized tensor through the vector path: quantize -> dequantize stays within half a step
+  w = torch.randn(4096, 4096, generator=g).bfloat16()
+  q = qd.quantize_per_tensor(w.cuda(), 0.05, 0, -128, 127, torch.int8)
+  assert torch.equal(q.cpu(), qd.quantize_per_tensor(w, 0.05, 0, -128, 127, torch.int8))
+  back = qd.dequantize_per_tensor(q, 0.05, 0, -128, 127, torch.int8).cpu()
+  inside = w.float().abs() <= 127 * 0.05
+  assert ((back - w.float()).abs()[inside] <= 0.025 + 1e-6).all()

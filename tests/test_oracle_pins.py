@@ -223,3 +223,52 @@ def test_reference_variants_cosine(n_bits, block, sym, qa):
   w, s, z = _rtn_like_reference(lin.weight.data, n_bits, block, sym)
   out = oracle.quantized_matmul(x, w, s, z, block_size=block, quantize_activation=qa)
   assert _cos(lin(x), out) > (0.97 if n_bits == 4 else 0.99)  # the reference asserts 0.99 on its seed
+
+
+# ---- quantized_decomposed quantize / dequantize (oracle/quantized_decomposed_oracle.py) -------------
+
+def _qdq_cases():
+  g = torch.Generator().manual_seed(5)
+  x = torch.randn(6, 10, 16, generator=g) * 3
+  x[0, 0, :8] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, 1e9, -1e9, 0.0])  # ties and saturation
+  return x
+
+
+def test_qdq_oracle_hand_values():
+  from oracle import quantized_decomposed_oracle as qo
+  # rint is half-to-even; zero point added after rounding; clamp last
+  q = qo.quantize_affine(np.array([0.5, 1.5, 2.5, -0.5, -1.5, 300.0, -300.0], dtype=np.float32), 1.0, 3, -128, 127,
+                         np.int8)
+  assert q.tolist() == [3, 5, 5, 3, 1, 127, -128]
+  assert qo.dequantize_per_tensor_f32(np.array([3, 5, -128], dtype=np.int8), 0.5, 3).tolist() == [0.0, 1.0, -65.5]
+  assert qo.dequantize_per_channel(np.array([[3, 5], [7, 9]], dtype=np.int8), [0.5, 2.0], [1, 2], 0).tolist() == \
+      [[1.0, 2.0], [10.0, 14.0]]
+
+
+def test_qdq_oracle_matches_torch_decomposition():
+  import torch.ao.quantization.fx._decomposed  # noqa: F401  (defines the CPU implementations)
+  from oracle import quantized_decomposed_oracle as qo
+  qd = torch.ops.quantized_decomposed
+  x = _qdq_cases()
+  for xdt in (torch.float32, torch.bfloat16, torch.float16):
+    xi = x.to(xdt)
+    for (scale, zp, lo, hi, dt, ndt) in [(0.037, -5, -128, 127, torch.int8, np.int8), (0.11, 128, 0, 255, torch.uint8, np.uint8),
+                                         (0.5, 0, -7, 7, torch.int8, np.int8), (0.01, 10, -32768, 32767, torch.int16, np.int16)]:
+      ref = qd.quantize_per_tensor(xi, scale, zp, lo, hi, dt)
+      inv = np.float32(1.0 / scale)
+      got = qo.quantize_affine(xi.float().numpy(), inv, zp, lo, hi, ndt)
+      assert np.array_equal(got, ref.numpy()), (xdt, scale)
+      deq = qd.dequantize_per_tensor(ref, scale, zp, lo, hi, dt)
+      assert np.array_equal(qo.dequantize_per_tensor_f32(ref.numpy(), scale, zp), deq.numpy())
+    for axis in (0, 1, 2):
+      c = x.shape[axis]
+      g = torch.Generator().manual_seed(axis)
+      scales = torch.rand(c, generator=g) * 0.1 + 0.01
+      zps = torch.randint(-20, 20, (c,), generator=g)
+      ref = qd.quantize_per_channel(xi, scales, zps, axis, -128, 127, torch.int8)
+      got = qo.quantize_affine(xi.float().numpy(), (1.0 / scales).numpy(), zps.numpy(), -128, 127, np.int8, axis)
+      assert np.array_equal(got, ref.numpy()), (xdt, axis)
+      deq = qd.dequantize_per_channel(ref, scales, zps, axis, -128, 127, torch.int8)
+      assert np.array_equal(qo.dequantize_per_channel(ref.numpy(), scales.numpy(), zps.numpy(), axis), deq.numpy())
+      deq0 = qd.dequantize_per_channel(ref, scales, None, axis, -128, 127, torch.int8)
+      assert np.array_equal(qo.dequantize_per_channel(ref.numpy(), scales.numpy(), None, axis), deq0.numpy())

@@ -15,6 +15,7 @@ OK, EINVAL, EUNSUPPORTED, EHIP = 0, -1, -2, -3
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 OVERFLOW_SATURATE, OVERFLOW_WRAP = 0, 1
 W_NK, W_SCN = 0, 1
+QDT_I8, QDT_U8, QDT_I16, QDT_I32 = 0, 1, 2, 3
 KERNEL_GENERIC, KERNEL_SKINNY_MFMA, KERNEL_W8A8_MFMA, KERNEL_W8A8_GENERIC = 0, 1, 2, 3
 ABI_VERSION = 2
 
@@ -36,6 +37,8 @@ SIGNATURES = {
     "xla_amd_qmm_w8a8_gemm": (_c_int, [_c_vp] * 8 + [_c_i64] * 3 + [_c_int] * 9 + [_c_vp]),
     "xla_amd_qmm_dispatch": (_c_int, [_c_i64] * 4 + [_c_int] * 3),
     "xla_amd_qmm_w8a8_tile": (_c_int, [_c_i64] * 3 + [ctypes.POINTER(ctypes.c_int32)]),
+    "xla_amd_qmm_quantize_affine": (_c_int, [_c_vp] * 4 + [_c_i64] * 3 + [_c_int] * 2 + [ctypes.c_int32] * 2 + [_c_vp]),
+    "xla_amd_qmm_dequantize_affine": (_c_int, [_c_vp] * 4 + [_c_i64] * 3 + [_c_int] * 3 + [_c_vp]),
 }
 
 _lib = None

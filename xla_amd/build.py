@@ -24,6 +24,7 @@ SOURCES = [
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=1"], "qmm_skinny_bf16.o"),
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=2"], "qmm_skinny_f16.o"),
     ("qmm_quant_act.hip", [], "qmm_quant_act.o"),
+    ("qmm_qdq.hip", [], "qmm_qdq.o"),
     ("qmm_w8a8_gemm.hip", [], "qmm_w8a8_gemm.o"),
 ]
 
