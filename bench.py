@@ -235,6 +235,24 @@ def main():
       _, ev, _ = time_calls([run_layer], 20, 5, use_graph)
       extra[f"llama3_8b_layer_linears_{tag}"] = {"us": round(ev * 1e3, 2),
                                                  "note": "weights (218 MB) stay cache-warm between iterations"}
+    # quantized_decomposed quantize / dequantize of a weight-sized tensor (HBM-bound elementwise)
+    import xla_amd.experimental.quantized  # noqa: F401
+    qd = torch.ops.quantized_decomposed
+    wf = [torch.randn(N_OUT, K_IN, generator=g5).bfloat16().to(dev) for _ in range(6)]  # 6 x 117 MB, rotating
+    _, ev_qt, _ = time_calls([(lambda t=t: qd.quantize_per_tensor(t, 0.05, 0, -128, 127, torch.int8)) for t in wf],
+                             24, 6, False)
+    qs = [qd.quantize_per_tensor(t, 0.05, 0, -128, 127, torch.int8) for t in wf]
+    _, ev_dq, _ = time_calls([(lambda t=t: qd.dequantize_per_tensor(t, 0.05, 0, -128, 127, torch.int8)) for t in qs],
+                             24, 6, False)
+    nel = N_OUT * K_IN
+    extra["quantized_decomposed_per_tensor_14336x4096"] = {
+        "quantize_bf16_to_int8_us": round(ev_qt * 1e3, 2),
+        "quantize_frac_hbm": round(nel * 3 / ev_qt / 1e6 / HBM_PEAK_GBPS, 4),
+        "dequantize_int8_to_f32_us": round(ev_dq * 1e3, 2),
+        "dequantize_frac_hbm": round(nel * 5 / ev_dq / 1e6 / HBM_PEAK_GBPS, 4),
+        "note": "eager calls (allocation and host-side parameter tensors included); bytes = read + written per element",
+    }
+    del wf, qs
     result["extra"] = extra
 
   # ---- CPU baseline: the oracle (reference's eager CPU semantics) on this host ----

@@ -77,25 +77,56 @@ qdq_quantize_kernel(const void* __restrict__ x, void* __restrict__ q, const floa
 
 // int_subtract != 0: out = cast(f32(q - zp[c]) * scale[c])            (per-channel form)
 // int_subtract == 0: out = round(round(cast(q) - zp[c]) * scale[c])   (per-tensor form, tensor ops in out's dtype)
+__device__ __forceinline__ float dequantize_value(int qv, int z, float sc, int out_dt, int int_subtract) {
+  if (int_subtract) return (float)(qv - z) * sc;
+  // (zero point and scale are host scalars there: they enter the arithmetic as f32)
+  const float a = qmm_round_dt((float)qv, out_dt);
+  const float d = qmm_round_dt(a - (float)z, out_dt);
+  return d * sc;
+}
+
+// VEC: one thread per 8 consecutive 1-byte elements of a row of `inner`
+// (inner % 8 == 0, 8-byte aligned q, 32-byte aligned out), else one per element.
+template <bool VEC>
 __global__ void __launch_bounds__(256)
 qdq_dequantize_kernel(const void* __restrict__ q, void* __restrict__ out, const float* __restrict__ scale,
                       const int32_t* __restrict__ zp, int64_t total, int64_t channels, int64_t inner,
                       int q_dt, int out_dt, int int_subtract) {
   const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= total) return;
-  const int64_t c = (t / inner) % channels;
-  const int qv = qdq_load_q(q, t, q_dt);
-  const int z = zp ? zp[c] : 0;
-  float r;
-  if (int_subtract) {
-    r = (float)(qv - z) * scale[c];
+  if constexpr (VEC) {
+    const int64_t e0 = t * 8;
+    if (e0 >= total) return;
+    const int64_t c = (e0 / inner) % channels;
+    const int z = zp ? zp[c] : 0;
+    const float sc = scale[c];
+    const i32x2 raw = *(const i32x2*)((const uint8_t*)q + e0);
+    float r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t b = ((uint32_t)raw[i >> 2] >> (8 * (i & 3))) & 0xffu;
+      const int qv = q_dt == XLA_AMD_QDT_I8 ? (int)(int8_t)b : (int)b;
+      r[i] = dequantize_value(qv, z, sc, out_dt, int_subtract);
+    }
+    if (out_dt == XLA_AMD_DT_F32) {
+      f32x4* o = (f32x4*)((float*)out + e0);
+      o[0] = f32x4{r[0], r[1], r[2], r[3]};
+      o[1] = f32x4{r[4], r[5], r[6], r[7]};
+    } else {
+      i32x4 pk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = out_dt == XLA_AMD_DT_BF16 ? qmm_f32_to_bf16(r[2 * i]) : qmm_f32_to_f16(r[2 * i]);
+        const uint32_t hi = out_dt == XLA_AMD_DT_BF16 ? qmm_f32_to_bf16(r[2 * i + 1]) : qmm_f32_to_f16(r[2 * i + 1]);
+        pk[i] = (int)(lo | (hi << 16));
+      }
+      *(i32x4*)((uint16_t*)out + e0) = pk;
+    }
   } else {
-    // (zero point and scale are host scalars there: they enter the arithmetic as f32)
-    const float a = qmm_round_dt((float)qv, out_dt);
-    const float d = qmm_round_dt(a - (float)z, out_dt);
-    r = d * scale[c];
+    if (t >= total) return;
+    const int64_t c = (t / inner) % channels;
+    const int z = zp ? zp[c] : 0;
+    qmm_store(out, t, dequantize_value(qdq_load_q(q, t, q_dt), z, scale[c], out_dt, int_subtract), out_dt);
   }
-  qmm_store(out, t, r, out_dt);
 }
 
 bool valid_qdt(int q_dt) { return q_dt >= XLA_AMD_QDT_I8 && q_dt <= XLA_AMD_QDT_I32; }
@@ -143,9 +174,16 @@ extern "C" int xla_amd_qmm_dequantize_affine(const void* q, void* out, const flo
   if (!qmm_valid_dt(out_dt) || !valid_qdt(q_dt)) return qmm_fail(XLA_AMD_QMM_EINVAL, "dequantize_affine: bad dtype enum");
   const int64_t total = outer * channels * inner;
   if (total == 0) return XLA_AMD_QMM_OK;
-  const int64_t blocks = (total + 255) / 256;
+  const bool vec = (q_dt == XLA_AMD_QDT_I8 || q_dt == XLA_AMD_QDT_U8) && inner % 8 == 0 &&
+                   (((uintptr_t)q & 7) == 0) && (((uintptr_t)out & 31) == 0);
+  const int64_t threads = vec ? total / 8 : total;
+  const int64_t blocks = (threads + 255) / 256;
   if (blocks > 0x7fffffffLL) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "dequantize_affine: tensor too large");
-  hipLaunchKernelGGL(qdq_dequantize_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, q, out, scale,
-                     zp, total, channels, inner, q_dt, out_dt, int_subtract);
+  if (vec)
+    hipLaunchKernelGGL(qdq_dequantize_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, q, out,
+                       scale, zp, total, channels, inner, q_dt, out_dt, int_subtract);
+  else
+    hipLaunchKernelGGL(qdq_dequantize_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, q, out,
+                       scale, zp, total, channels, inner, q_dt, out_dt, int_subtract);
   return QMM_CHECK_LAUNCH("dequantize_affine launch");
 }

@@ -38,6 +38,15 @@ def _check_scale_zp(input, scale, zero_point, axis, dtype):
   assert bool((scale > 0).all())
 
 
+def _check_scalar(scale, zero_point, dtype):
+  # the same conditions for host scalars
+  assert 'int' in str(dtype)
+  assert dtype in _QDT, f"xla_amd: quantized dtype {dtype} is not supported on the GPU path"
+  info = torch.iinfo(dtype)
+  assert info.min <= zero_point <= info.max
+  assert scale > 0
+
+
 def _geometry(input, axis, n_params):
   """[outer, channels, inner] view of a contiguous tensor for parameters along `axis`."""
   if axis == -1 or n_params == 1:
@@ -81,6 +90,23 @@ def _dequantize(input, scale, zero_point, dtype, out_dtype, axis, int_subtract):
   return out
 
 
+# per-tensor parameters are host scalars: their one-element device tensors are kept, so that a call
+# does not pay two host-to-device copies
+_scalar_cache = {}
+
+
+def _scalar_params(device, a: float, z: int):
+  key = (str(device), a, z)
+  hit = _scalar_cache.get(key)
+  if hit is None:
+    if len(_scalar_cache) > 256:
+      _scalar_cache.clear()
+    hit = (torch.tensor([a], dtype=torch.float64).to(torch.float32).to(device),
+           torch.tensor([z], dtype=torch.int32).to(device))
+    _scalar_cache[key] = hit
+  return hit
+
+
 def _float_input(input):
   assert input.dtype in (torch.float32, torch.bfloat16, torch.float16), \
       f"Expecting input to have dtype torch.float32, but got dtype: {input.dtype}"
@@ -90,11 +116,10 @@ def _float_input(input):
 def rocm_quantize_per_tensor(input: torch.Tensor, scale: float, zero_point: int, quant_min: int, quant_max: int,
                              dtype: torch.dtype):
   _float_input(input)
-  scale_t = torch.tensor([scale], dtype=torch.float64)
-  _check_scale_zp(input, scale_t, torch.tensor([zero_point], dtype=torch.int64), -1, dtype)
+  _check_scalar(scale, zero_point, dtype)
   # torch: inv_scale = 1.0 / scale in double, then multiplied into an f32 tensor as an f32 scalar
-  inv = torch.tensor([1.0 / scale], dtype=torch.float64).to(torch.float32)
-  return _quantize(input, inv, torch.tensor([zero_point]), quant_min, quant_max, dtype, -1)
+  inv, zp = _scalar_params(input.device, 1.0 / scale, zero_point)
+  return _quantize(input, inv, zp, quant_min, quant_max, dtype, -1)
 
 
 @impl(quantized_decomposed_lib, "quantize_per_channel", "CUDA")
@@ -110,10 +135,9 @@ def rocm_quantize_per_channel(input: torch.Tensor, scales: torch.Tensor, zero_po
 @impl(quantized_decomposed_lib, "dequantize_per_tensor", "CUDA")
 def rocm_dequantize_per_tensor(input: torch.Tensor, scale: float, zero_point: int, quant_min: int, quant_max: int,
                                dtype: torch.dtype, *, out_dtype=None):
-  _check_scale_zp(input, torch.tensor([scale], dtype=torch.float64), torch.tensor([zero_point], dtype=torch.int64), -1,
-                  dtype)
-  return _dequantize(input, torch.tensor([scale], dtype=torch.float64).to(torch.float32), torch.tensor([zero_point]),
-                     dtype, out_dtype, -1, 0)
+  _check_scalar(scale, zero_point, dtype)
+  sc, zp = _scalar_params(input.device, scale, zero_point)
+  return _dequantize(input, sc, zp, dtype, out_dtype, -1, 0)
 
 
 @impl(quantized_decomposed_lib, "dequantize_per_channel", "CUDA")
