@@ -327,16 +327,16 @@ def test_tile_weight_layout(ops):
 
 def test_w8a8_tiles_and_tails(ops):
   # every workgroup tile the kernel offers, on shapes with M/N/K tails
-  for bm in (64, 128, 256):
-    for (m, n, k) in [(bm + 3, 2 * bm + 5, 144), (17, 33, 64), (bm, bm, 4096)]:
+  for bm, bn in ((64, 64), (128, 128), (128, 256), (256, 256)):
+    for (m, n, k) in [(bm + 3, 2 * bn + 5, 144), (17, 33, 64), (bm, bn, 4096)]:
       g = cases.gen(bm + m + n)
       xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
       w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
       _, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), torch.ones(m, 1).cuda(), torch.ones(n).cuda(), None, None,
                                  cvt_dtype=torch.float32, mid_dtype=torch.float32, out_dtype=torch.float32,
-                                 want_acc=True, block_m=bm, block_n=bm)
+                                 want_acc=True, block_m=bm, block_n=bn)
       ref = torch.from_numpy(xq.numpy().astype(np.int64) @ w.numpy().astype(np.int64).T)
-      assert torch.equal(acc.cpu().long(), ref), (bm, m, n, k)
+      assert torch.equal(acc.cpu().long(), ref), (bm, bn, m, n, k)
 
 
 def test_w8a8_column_split_two_tile_widths(ops):

@@ -401,6 +401,7 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 static void choose_tile(int64_t M, int64_t N, int* bm, int* bn) {
   auto tiles = [&](int a, int b) { return ((M + a - 1) / a) * ((N + b - 1) / b); };
   if (M > 128 && N > 128 && tiles(256, 256) >= 200) { *bm = 256; *bn = 256; return; }
+  if (M > 64 && N > 128 && tiles(128, 256) >= 160) { *bm = 128; *bn = 256; return; }
   if (M > 64 && tiles(128, 128) >= 128) { *bm = 128; *bn = 128; return; }
   *bm = 64; *bn = 64;
 }
@@ -486,6 +487,7 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
     }
     return rc;
   }
+  if (bm == 128 && bn == 256) return launch_tile<128, 256, 2, 4>(g, s);  // 8 waves, wave tile 64 x 64
   if (bm == 128 && bn == 128) return launch_tile<128, 128, 2, 2>(g, s);
   if (bm == 64 && bn == 64) return launch_tile<64, 64, 2, 2>(g, s);
   return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_gemm: no kernel for tile %dx%d", bm, bn);
