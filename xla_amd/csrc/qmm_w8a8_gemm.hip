@@ -456,7 +456,7 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
     // 256 x 192 tiles takes 3/4 of a round of 256 x 256 tiles).  cfg4 (2048 x 14336):
     // 8 x 56 = 448 tiles = 2 rounds becomes 8 x 32 + 8 x 32 = 1 + 0.75 rounds.
     int64_t best_n1 = (N + 255) / 256;
-    if (block_m == 0 && block_n == 0) {
+    {
       const int64_t mt = (M + 255) / 256;
       auto rounds = [](int64_t tiles) { return (double)((tiles + 255) / 256); };
       double best = rounds(mt * best_n1);

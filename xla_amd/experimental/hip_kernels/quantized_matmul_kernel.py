@@ -26,7 +26,9 @@ def _add(batches, n_out, n_in, blocks):
 for _n_out, _n_in in ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (6144, 4096),
                       (28672, 4096)):
   _add((1024, 2048, 4096, 8192), _n_out, _n_in, (256, 256, 128))
-  _add((256, 512), _n_out, _n_in, (128, 128, 128))
+  # (128 x 256 once it still gives >= 160 workgroups)
+  _add((512,), _n_out, _n_in, (128, 256, 128) if _n_out >= 10240 else (128, 128, 128))
+  _add((256,), _n_out, _n_in, (128, 256, 128) if _n_out >= 20480 else (128, 128, 128))
   _add((64, 128), _n_out, _n_in, (64, 64, 128))
 
 
