@@ -111,7 +111,9 @@ def test_config3_blockwise(ops, bits, int4, sym):
 @pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("bits", [4, 8])
 def test_blockwise_shapes(ops, xdt, bits):
-  for (m, n, k, c) in [(2, 24, 256, 128), (19, 40, 512, 256), (3, 8, 6, 2), (5, 16, 96, 32)]:
+  # (n = 22: no 16-byte scale loads, generic kernel; k = 8192: the x columns are replaced mid-way, k-split waves)
+  for (m, n, k, c) in [(2, 24, 256, 128), (19, 40, 512, 256), (3, 8, 6, 2), (5, 16, 96, 32), (4, 22, 256, 128),
+                       (16, 256, 8192, 128), (20, 4096, 2048, 512)]:
     x, w, s, z, _ = cases.blockwise(m, n, k, c, bits, xdt, symmetric=False, seed=m)
     exp = oracle.quantized_matmul(x, w, s, z, block_size=c)
     out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=c, int4_weight=(bits == 4))
