@@ -138,7 +138,8 @@ constexpr int kRedNone = 0;    // blockwise, KW == 1: nothing to reduce
 constexpr int kRedRaw = 1;     // per-channel (C == K, any KW): raw dot products and x sums are summed, then scaled
 constexpr int kRedScaled = 2;  // blockwise, KW > 1, whole blocks per step (KS % C == 0): scaled block results are summed
 
-// NW waves per workgroup; WSEG weight bytes per row per step.
+// NW waves per workgroup; WSEG weight bytes per row per step.  Every launch uses the defaults
+// (4 waves, 512 bytes); an 8-wave shape with 256-byte steps measured slower and is not dispatched.
 template <int XT, int BITS, int MT, int KW, int NW = kWaves, int WSEG = kWSeg>
 struct SkinnyCfg {
   static constexpr int RW = NW / KW;
@@ -547,7 +548,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // ---- reduction over k-splits, final rounding, store ------------------------------------
   const int zpo_dt = qmm_promote(x_dt, a.zp_dt);
   if constexpr (KW > 1) {
-    __syncthreads();  // pipeline stages are dead: reuse LDS
+    __syncthreads();  // every wave is done with the x tiles: reuse LDS
     float* red = (float*)smem;  // [KW][RW][slot][64]
     constexpr int kSlots = RED == kRedRaw ? 4 * MT + (NEEDXS ? MT : 0) : (HASZP ? 8 * MT : 4 * MT);
     float* mine = red + ((kw * RW + rw) * kSlots) * 64 + lane;
