@@ -235,6 +235,22 @@ def main():
       _, ev, _ = time_calls([run_layer], 20, 5, use_graph)
       extra[f"llama3_8b_layer_linears_{tag}"] = {"us": round(ev * 1e3, 2),
                                                  "note": "weights (218 MB) stay cache-warm between iterations"}
+
+      # the same layer with q/k/v and gate/up concatenated along N: 4 launches instead of 7
+      def cat(names):
+        return (torch.cat([layer_s[n][0] for n in names]).contiguous(),
+                torch.cat([layer_s[n][1] for n in names]).contiguous())
+
+      fused_s = {"qkv": cat(("q", "k", "v")), "o": layer_s["o"], "gate_up": cat(("gate", "up")),
+                 "down": layer_s["down"]}
+
+      def run_fused():
+        for name, (w, s) in fused_s.items():
+          op(x_in[w.shape[1]], w, s, quantize_activation=qa)
+
+      _, ev, _ = time_calls([run_fused], 20, 5, use_graph)
+      extra[f"llama3_8b_layer_linears_{tag}"]["us_qkv_and_gate_up_fused"] = round(ev * 1e3, 2)
+      del fused_s
     # quantized_decomposed quantize / dequantize of a weight-sized tensor (HBM-bound elementwise)
     import xla_amd.experimental.quantized  # noqa: F401
     qd = torch.ops.quantized_decomposed

@@ -435,3 +435,18 @@ def test_qdq_ops_match_oracle_and_torch_cpu(ops):
   back = qd.dequantize_per_tensor(q, 0.05, 0, -128, 127, torch.int8).cpu()
   inside = w.float().abs() <= 127 * 0.05
   assert ((back - w.float()).abs()[inside] <= 0.025 + 1e-6).all()
+
+
+def test_fused_linears_on_gpu(ops):
+  # q/k/v-style N-concatenation: one launch, outputs identical to the separate layers
+  from xla_amd.quantization import quantize_linear, fuse_quantized_linears
+  torch.manual_seed(11)
+  for kwargs, xdt in ((dict(n_bits=8, scale_dtype=torch.bfloat16), torch.bfloat16),
+                      (dict(n_bits=8, quantize_activation=True), torch.bfloat16),
+                      (dict(n_bits=4, block_size=128, symmetric=False, scale_dtype=torch.bfloat16), torch.bfloat16)):
+    lins = [quantize_linear(torch.nn.Linear(512, n, bias=False), **kwargs).cuda() for n in (256, 64, 128)]
+    fused = fuse_quantized_linears(lins)
+    x = torch.randn(9, 512).to(xdt).cuda()
+    outs = fused(x).split([l.output_dim for l in lins], dim=-1)
+    for l, o in zip(lins, outs):
+      assert torch.equal(l(x), o), kwargs

@@ -184,3 +184,17 @@ def test_product_does_not_import_the_oracle():
       if f.endswith((".py", ".hip", ".h", ".cpp")):
         text = open(os.path.join(dirpath, f)).read()
         assert "oracle" not in text.lower().replace("no fallback", ""), f"{f} mentions the oracle"
+
+
+def test_fuse_quantized_linears_cpu():
+  # N-concatenated layers give exactly the outputs of the separate layers (CPU operator path)
+  import xla_amd.experimental.custom_kernel  # noqa: F401
+  from xla_amd.quantization import quantize_linear, fuse_quantized_linears
+  torch.manual_seed(3)
+  x = torch.randn(5, 64)
+  for kwargs in (dict(n_bits=8), dict(n_bits=8, symmetric=False), dict(n_bits=4, block_size=32, symmetric=False)):
+    lins = [quantize_linear(torch.nn.Linear(64, n, bias=False), **kwargs) for n in (24, 8, 16)]
+    fused = fuse_quantized_linears(lins)
+    outs = fused(x).split([l.output_dim for l in lins], dim=-1)
+    for l, o in zip(lins, outs):
+      assert torch.equal(l(x), o), kwargs

@@ -83,3 +83,34 @@ def replace_linear_with_quantized(module: torch.nn.Module, predicate=None, **kwa
     else:
       replace_linear_with_quantized(child, predicate, **kwargs)
   return module
+
+
+def fuse_quantized_linears(linears) -> XlaQuantizedLinear:
+  """One XlaQuantizedLinear that computes several of them side by side.
+
+  The layers must read the same input (same in_features) and share their
+  quantization settings; their output channels are concatenated in the order
+  given, so `fused(x).split([l.output_dim for l in linears], dim=-1)` equals
+  `[l(x) for l in linears]` exactly (every output channel keeps its own weight
+  row, scale and zero point).  Meant for the q/k/v and gate/up pairs of a
+  decoder layer: one launch streams all the weights, instead of one launch
+  (with its fixed cost) per projection.
+  """
+  linears = list(linears)
+  first = linears[0]
+  for l in linears[1:]:
+    assert (l.input_dim, l.is_symmetric, l.block_size, l.int4_weight, l.quantize_activation) == \
+        (first.input_dim, first.is_symmetric, first.block_size, first.int4_weight, first.quantize_activation), \
+        "fused layers must share input size and quantization settings"
+    assert l.weight.dtype == first.weight.dtype and l.weight_scaler.dtype == first.weight_scaler.dtype
+  out_dim = sum(l.output_dim for l in linears)
+  fused = XlaQuantizedLinear(first.input_dim, out_dim, first.is_symmetric, first.block_size, first.int4_weight,
+                             first.quantize_activation)
+  cat_dim = 0 if first.block_size == -1 else -1  # per-channel [out, in] / [out]; blockwise [.., out]
+  weight = torch.cat([l.weight for l in linears], dim=cat_dim).contiguous()
+  scaler = torch.cat([l.weight_scaler for l in linears], dim=cat_dim).contiguous()
+  zero_point = None
+  if first.zero_point is not None:
+    zero_point = torch.cat([l.zero_point for l in linears], dim=cat_dim).contiguous()
+  fused.load_quantized_weight(weight, scaler, zero_point)
+  return fused
