@@ -281,16 +281,18 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
           const float v0 = ((float)a[0] * ws[0]) * xs, v1 = ((float)a[1] * ws[1]) * xs;
           const float v2 = ((float)a[2] * ws[2]) * xs, v3 = ((float)a[3] * ws[3]) * xs;
           const size_t idx0 = (size_t)(m0 + rbase + row) * g.ldo + (n0 + wn * TN + c4 * 4);
+          // (streaming stores: the output is written once and not read here, it should
+          // not push the operands out of L2)
           if constexpr (EPI == 3) {
-            *(f32x4*)((float*)g.out + idx0) = f32x4{v0, v1, v2, v3};
+            __builtin_nontemporal_store(f32x4{v0, v1, v2, v3}, (f32x4*)((float*)g.out + idx0));
           } else if constexpr (EPI == 1) {
             const uint32_t lo = qmm_f32_to_bf16(v0) | ((uint32_t)qmm_f32_to_bf16(v1) << 16);
             const uint32_t hi = qmm_f32_to_bf16(v2) | ((uint32_t)qmm_f32_to_bf16(v3) << 16);
-            *(i32x2*)((uint16_t*)g.out + idx0) = i32x2{(int)lo, (int)hi};
+            __builtin_nontemporal_store(i32x2{(int)lo, (int)hi}, (i32x2*)((uint16_t*)g.out + idx0));
           } else {
             const uint32_t lo = qmm_f32_to_f16(v0) | ((uint32_t)qmm_f32_to_f16(v1) << 16);
             const uint32_t hi = qmm_f32_to_f16(v2) | ((uint32_t)qmm_f32_to_f16(v3) << 16);
-            *(i32x2*)((uint16_t*)g.out + idx0) = i32x2{(int)lo, (int)hi};
+            __builtin_nontemporal_store(i32x2{(int)lo, (int)hi}, (i32x2*)((uint16_t*)g.out + idx0));
           }
         }
       });
