@@ -343,13 +343,13 @@ def test_w8a8_tiles_and_tails(ops):
 
 def test_w8a8_column_split_two_tile_widths(ops):
   # a shape whose 256-wide tiles would leave the last round of workgroups mostly empty: the library covers the
-  # columns with 256-wide and 192-wide tiles in two launches; ragged last tile, partial last K step
-  m, n, k = 2048, 14436, 192
+  # columns with 32 256-wide and 32 192-wide tiles in two launches; ragged last tile, partial last K step
+  m, n, k = 2048, 14300, 1088
   g = cases.gen(99)
   xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
   w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
   xs, ws = torch.rand(m, 1, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
-  ref = torch.from_numpy(xq.numpy().astype(np.int64) @ w.numpy().astype(np.int64).T)
+  ref = (xq.double() @ w.double().T).long()  # exact: |sum| < 2^53
   out, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), xs.cuda(), ws.cuda(), None, None, cvt_dtype=torch.float32,
                                mid_dtype=torch.float32, out_dtype=torch.float32, want_acc=True)
   assert torch.equal(acc.cpu().long(), ref)

@@ -398,20 +398,56 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 
 }  // namespace
 
-// Tile choice by shape: big tiles when the grid still fills 256 CUs, smaller
-// ones for small problems.
-static void choose_tile(int64_t M, int64_t N, int* bm, int* bn) {
+// Estimated time in us of the launches that cover an output, fitted to measurements at
+// K = 128 ... 14336: a launch costs kLaunchUs, and each round of tiles over the 256 CUs
+// costs a part per tile (prologue, epilogue) plus a part proportional to K.  A round
+// that is only partly full costs a whole one.
+struct TileCost { double per_round_us, per_k4096_us; };
+static constexpr double kLaunchUs = 4.0;
+static constexpr TileCost kCost256 = {11.0, 52.0}, kCost192 = {8.0, 39.0}, kCost128x256 = {9.0, 27.0},
+                          kCost128 = {8.0, 14.0};
+static double rounds_us(const TileCost& c, int64_t tiles, int64_t K) {
+  return (double)((tiles + 255) / 256) * (c.per_round_us + c.per_k4096_us * (double)K / 4096.0);
+}
+
+// Columns covered by n1 tiles of 256 followed by n2 tiles of 192 (two launches when
+// both are present): the split with the least estimated time.  2048 x 14336:
+// 8 x 56 = 448 tiles = 2 rounds becomes 8 x 32 + 8 x 32 = 1 + 0.75 rounds.
+static double best_column_split(int64_t M, int64_t N, int64_t K, int64_t* n1_out) {
+  const int64_t mt = (M + 255) / 256;
+  int64_t best_n1 = (N + 255) / 256;
+  double best = kLaunchUs + rounds_us(kCost256, mt * best_n1, K);
+  for (int64_t n1 = N / 256; n1 >= 0; --n1) {
+    const int64_t n2 = (N - n1 * 256 + 191) / 192;
+    if (n2 <= 0) continue;
+    const double cost = (n1 > 0 ? 2 : 1) * kLaunchUs + rounds_us(kCost256, mt * n1, K) +
+                        rounds_us(kCost192, mt * n2, K);
+    if (cost < best - 1e-9) { best = cost; best_n1 = n1; }
+  }
+  *n1_out = best_n1;
+  return best;
+}
+
+// Tile choice by shape: 64 x 64 tiles (several workgroups resident per CU, which hides
+// the latency of their short K steps) while there are fewer than four per CU: measured
+// faster than one round of 128 x 128 tiles up to there, for K = 2048 ... 14336.  Larger
+// problems take the tile class with the least estimated time.
+static void choose_tile(int64_t M, int64_t N, int64_t K, int* bm, int* bn) {
   auto tiles = [&](int a, int b) { return ((M + a - 1) / a) * ((N + b - 1) / b); };
-  if (M > 128 && N > 128 && tiles(256, 256) >= 200) { *bm = 256; *bn = 256; return; }
-  if (M > 64 && N > 128 && tiles(128, 256) >= 160) { *bm = 128; *bn = 256; return; }
-  if (M > 64 && tiles(128, 128) >= 128) { *bm = 128; *bn = 128; return; }
-  *bm = 64; *bn = 64;
+  if (M <= 64 || tiles(64, 64) < 1024) { *bm = 64; *bn = 64; return; }
+  int64_t n1;
+  const double c256 = M > 128 && N > 128 ? best_column_split(M, N, K, &n1) : 1e30;
+  const double c128x256 = N > 128 ? kLaunchUs + rounds_us(kCost128x256, tiles(128, 256), K) : 1e30;
+  const double c128 = kLaunchUs + rounds_us(kCost128, tiles(128, 128), K);
+  if (c256 <= c128x256 && c256 <= c128) { *bm = 256; *bn = 256; return; }
+  if (c128x256 <= c128) { *bm = 128; *bn = 256; return; }
+  *bm = 128; *bn = 128;
 }
 
 extern "C" int xla_amd_qmm_w8a8_tile(int64_t M, int64_t N, int64_t K, int32_t* tile_mnk) {
   if (!tile_mnk || M <= 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_tile: bad arguments");
   int bm, bn;
-  choose_tile(M, N, &bm, &bn);
+  choose_tile(M, N, K, &bm, &bn);
   tile_mnk[0] = bm; tile_mnk[1] = bn; tile_mnk[2] = kBK;
   return XLA_AMD_QMM_OK;
 }
@@ -448,27 +484,12 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
   g.mid_dt = mid_dt; g.zpo_dt = zpo_dt; g.out_dt = out_dt;
   g.tiles_m = g.tiles_n = 0;
   int bm = block_m, bn = block_n;
-  if (bm == 0 && bn == 0) choose_tile(M, N, &bm, &bn);
+  if (bm == 0 && bn == 0) choose_tile(M, N, K, &bm, &bn);
   // 256x256: 8 waves (2 x 4, wave tile 128 x 64): two waves per SIMD, so that one wave's LDS and
   // barrier waits are the other's MFMA slots (measured 128 us against 154 us with 4 waves of 128 x 128)
   if (bm == 256 && bn == 256) {
-    // Rounds of tiles over the 256 CUs: a last round that is only partly full costs a
-    // whole round.  Columns can be covered by n1 tiles of 256 followed by n2 tiles of
-    // 192 (two launches); pick the split with the least estimated time (a round of
-    // 256 x 192 tiles takes 3/4 of a round of 256 x 256 tiles).  cfg4 (2048 x 14336):
-    // 8 x 56 = 448 tiles = 2 rounds becomes 8 x 32 + 8 x 32 = 1 + 0.75 rounds.
-    int64_t best_n1 = (N + 255) / 256;
-    {
-      const int64_t mt = (M + 255) / 256;
-      auto rounds = [](int64_t tiles) { return (double)((tiles + 255) / 256); };
-      double best = rounds(mt * best_n1);
-      for (int64_t n1 = N / 256; n1 >= 0; --n1) {
-        const int64_t n2 = (N - n1 * 256 + 191) / 192;
-        if (n2 <= 0) continue;
-        const double cost = rounds(mt * n1) + 0.75 * rounds(mt * n2) + (n1 > 0 ? 0.02 : 0.0);
-        if (cost < best - 1e-9) { best = cost; best_n1 = n1; }
-      }
-    }
+    int64_t best_n1;
+    best_column_split(M, N, K, &best_n1);
     const int64_t N1 = best_n1 * 256 < N ? best_n1 * 256 : N;
     int rc = XLA_AMD_QMM_OK;
     if (N1 > 0) {

@@ -22,14 +22,31 @@ def _add(batches, n_out, n_in, blocks):
       TUNED_BLOCK_SIZES[(_ARCH, bs, n_out, n_in, dtype, True)] = blocks
 
 
-# Llama-3-8B linears (q/o, k/v, gate/up, down) at prefill batch sizes.
-for _n_out, _n_in in ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (6144, 4096),
-                      (28672, 4096)):
-  _add((1024, 2048, 4096, 8192), _n_out, _n_in, (256, 256, 128))
-  # (128 x 256 once it still gives >= 160 workgroups)
-  _add((512,), _n_out, _n_in, (128, 256, 128) if _n_out >= 10240 else (128, 128, 128))
-  _add((256,), _n_out, _n_in, (128, 256, 128) if _n_out >= 20480 else (128, 128, 128))
-  _add((64, 128), _n_out, _n_in, (64, 64, 128))
+# Fastest measured tile per shape (MI355X, one sweep over the four tile classes; ties
+# within 3 % go to what the library would pick by itself).  Shapes: the Llama-3-8B
+# linears (q/o, k/v, gate+up fused and single, qkv fused, down) and two square ones.
+# (n_out, n_in): {batch: (batch_block, out_block)}
+_MEASURED = {
+    (4096, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (128, 128),
+                   2048: (128, 256), 4096: (256, 256), 8192: (256, 256)},
+    (1024, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (64, 64),
+                   2048: (64, 64), 4096: (64, 64), 8192: (128, 256)},
+    (14336, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (128, 256), 1024: (256, 256),
+                    2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
+    (4096, 14336): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (128, 128),
+                    2048: (128, 256), 4096: (256, 256), 8192: (256, 256)},
+    (6144, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (128, 256),
+                   2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
+    (28672, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (128, 256), 512: (256, 256), 1024: (256, 256),
+                    2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
+    (8192, 8192): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (128, 128), 1024: (128, 256),
+                   2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
+    (2048, 2048): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (64, 64),
+                   2048: (64, 64), 4096: (128, 256), 8192: (256, 256)},
+}
+for (_n_out, _n_in), _by_batch in _MEASURED.items():
+  for _bs, (_bm, _bn) in _by_batch.items():
+    _add((_bs,), _n_out, _n_in, (_bm, _bn, 128))
 
 
 def get_device_arch(device=None) -> str:
