@@ -341,6 +341,21 @@ def test_w8a8_tiles_and_tails(ops):
       assert torch.equal(acc.cpu().long(), ref), (bm, bn, m, n, k)
 
 
+def test_w8a8_pipeline_depths_and_k_steps(ops):
+  # 64 x 64 tiles run with three LDS stages up to 512 tiles and with two above; K from less than one
+  # step (128) to several, with and without a partial last step, crosses every prologue/drain case
+  for (m, n) in ((70, 130), (64 * 24, 64 * 24)):  # 6 tiles, 576 tiles
+    for k in (16, 112, 128, 144, 256, 272, 384, 400, 1040):
+      g = cases.gen(m + k)
+      xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+      w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+      _, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), torch.ones(m, 1).cuda(), torch.ones(n).cuda(), None, None,
+                                 cvt_dtype=torch.float32, mid_dtype=torch.float32, out_dtype=torch.float32,
+                                 want_acc=True, block_m=64, block_n=64)
+      ref = (xq.double() @ w.double().T).long()  # exact: |sum| < 2^53
+      assert torch.equal(acc.cpu().long(), ref), (m, n, k)
+
+
 def test_w8a8_column_split_two_tile_widths(ops):
   # a shape whose 256-wide tiles would leave the last round of workgroups mostly empty: the library covers the
   # columns with 32 256-wide and 32 192-wide tiles in two launches; ragged last tile, partial last K step

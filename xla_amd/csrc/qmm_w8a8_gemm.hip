@@ -48,7 +48,13 @@ __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >>
 // accumulator output, partial tiles); 1/2/3 = all-f32 scale chain with bf16 /
 // f16 / f32 output and nothing else, which whole tiles finish with a short
 // branch-free loop (partial tiles of such a launch still take the general code).
-template <int BM, int BN, int WM, int WN, int EPI>
+// s_waitcnt immediate for "at most n vector-memory operations outstanding" (n < 64),
+// leaving expcnt and lgkmcnt alone
+constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
+
+// NS = LDS pipeline stages: the copies of NS - 1 K steps are in flight while one is
+// computed.
+template <int BM, int BN, int WM, int WN, int EPI, int NS>
 __global__ void __launch_bounds__(WM * WN * 64)
 qmm_w8a8_gemm_kernel(GemmArgs g) {
   constexpr int T = WM * WN * 64;
@@ -58,8 +64,8 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be a multiple of 32");
   static_assert((BM * 8) % T == 0 && (BN * 8) % T == 0, "tile rows must divide over the threads");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* sA = smem;                      // [2][BM][128]
-  char* sB = smem + 2 * BM * kBK;       // [2][BN][128]
+  char* sA = smem;                      // [NS][BM][128]
+  char* sB = smem + NS * BM * kBK;      // [NS][BN][128]
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases in scalar registers
@@ -131,11 +137,18 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
       });
     }
   };
-  // All of this wave's copies have landed in LDS (they count as vector-memory
-  // operations), then the workgroup meets.
-  auto stage_sync = [&]() __attribute__((always_inline)) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), leave expcnt/lgkmcnt alone
-    qmm_lds_barrier();
+  // This wave's copies of a stage have landed in LDS (they count as vector-memory
+  // operations, which complete in order: at most the copies of the `later` full
+  // stages issued after it may be outstanding), then the workgroup meets.
+  constexpr int kStageOps = A_CH + B_CH;
+  static_assert((NS - 2) * kStageOps < 64, "vmcnt is a 6-bit counter");
+  // (A workgroup-scope release fence would make the compiler wait for every copy in
+  // flight, since the copies are LDS writes; the asm barrier with a memory clobber keeps
+  // the order of the LDS accesses around it, and the explicit counts do the waiting.)
+  auto stage_sync = [&](bool later_stages_all_full) __attribute__((always_inline)) {
+    if (NS > 2 && later_stages_all_full) __builtin_amdgcn_s_waitcnt(vmcnt_imm((NS - 2) * kStageOps));
+    else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   };
 
   // Scales of this tile are fetched now so that their latency is hidden by the
@@ -207,16 +220,23 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
     });
   };
 
+  // Steps 0 .. NS-2 are copied ahead; step kt then computes stage kt % NS while the
+  // copy of step kt + NS - 1 goes into the stage that step kt - 1 read, which every
+  // wave has left at the barrier of step kt.  When step kt is waited for, the steps
+  // issued after it are kt+1 .. min(kt + NS - 2, last): they are NS - 2 full stages
+  // unless they include the last step, which may be partial (fewer copies per wave).
   const int ksteps = (K + kBK - 1) / kBK;
-  stage_load(0, 0);
-  stage_sync();
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < ksteps) stage_load(s, s * kBK);
+  int cur = 0, nxt = NS - 1;
   for (int kt = 0; kt < ksteps; ++kt) {
-    const int cur = kt & 1;
-    // stage cur^1 was last read in step kt-1, which every wave has left
+    stage_sync(kt + NS - 2 < ksteps - 1);
     compute(cur, [&]() __attribute__((always_inline)) {
-      if (kt + 1 < ksteps) stage_load(cur ^ 1, (kt + 1) * kBK);
+      if (kt + NS - 1 < ksteps) stage_load(nxt, (kt + NS - 1) * kBK);
     });
-    stage_sync();
+    cur = cur + 1 == NS ? 0 : cur + 1;
+    nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
 
   // Epilogue, staged through LDS so that (a) the code stays small (the
@@ -225,7 +245,7 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   // stores are row-contiguous vectors instead of one element per lane.
   constexpr int kEpStride = TN + 8;  // ints per staged row: +8 keeps rows 16-byte aligned and
                                      // shifts the second half-wave (4 rows down) by 32 banks
-  static_assert(4 * WM * WN * 32 * kEpStride + 4 * 4 * (BM + BN) <= 2 * (BM + BN) * kBK,
+  static_assert(4 * WM * WN * 32 * kEpStride + 4 * 4 * (BM + BN) <= NS * (BM + BN) * kBK,
                 "epilogue staging must fit in the pipeline's LDS");
   __syncthreads();  // every wave is done reading the last pipeline stage
   float* s_xs = (float*)smem;          // [BM] activation scale
@@ -364,15 +384,15 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   });
 }
 
-template <int BM, int BN, int WM, int WN, int EPI>
+template <int BM, int BN, int WM, int WN, int EPI, int NS>
 int launch_tile_epi(GemmArgs g, hipStream_t stream) {
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   const int ntiles = g.tiles_m * g.tiles_n;
   const int per = (ntiles + 7) / 8;
   const unsigned grid = (unsigned)(per * 8);
-  constexpr size_t lds = 2 * (size_t)(BM + BN) * kBK;
-  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN, EPI>;
+  constexpr size_t lds = NS * (size_t)(BM + BN) * kBK;
+  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN, EPI, NS>;
   static thread_local bool attr_set = false;
   if (!attr_set) {
     int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
@@ -386,14 +406,14 @@ int launch_tile_epi(GemmArgs g, hipStream_t stream) {
 
 // The short epilogue applies when the scale chain is all f32, there is no zero
 // point, no raw-accumulator output and rows of out are vector-aligned.
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS = 2>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const bool fast = g.out && !g.acc_out && !g.zp && g.cvt_dt == XLA_AMD_DT_F32 &&
                     g.mid_dt == XLA_AMD_DT_F32 && (g.N % 4) == 0 && (g.ldo % 4) == 0 && (((uintptr_t)g.out) & 15) == 0;
-  if (fast && g.out_dt == XLA_AMD_DT_BF16) return launch_tile_epi<BM, BN, WM, WN, 1>(g, stream);
-  if (fast && g.out_dt == XLA_AMD_DT_F16) return launch_tile_epi<BM, BN, WM, WN, 2>(g, stream);
-  if (fast && g.out_dt == XLA_AMD_DT_F32) return launch_tile_epi<BM, BN, WM, WN, 3>(g, stream);
-  return launch_tile_epi<BM, BN, WM, WN, 0>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_BF16) return launch_tile_epi<BM, BN, WM, WN, 1, NS>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_F16) return launch_tile_epi<BM, BN, WM, WN, 2, NS>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_F32) return launch_tile_epi<BM, BN, WM, WN, 3, NS>(g, stream);
+  return launch_tile_epi<BM, BN, WM, WN, 0, NS>(g, stream);
 }
 
 }  // namespace
@@ -512,6 +532,13 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
   }
   if (bm == 128 && bn == 256) return launch_tile<128, 256, 2, 4>(g, s);  // 8 waves, wave tile 64 x 64
   if (bm == 128 && bn == 128) return launch_tile<128, 128, 2, 2>(g, s);
-  if (bm == 64 && bn == 64) return launch_tile<64, 64, 2, 2>(g, s);
+  if (bm == 64 && bn == 64) {
+    // Up to two workgroups per CU there is little else on a CU to cover the latency of a
+    // K step's copies with, and a 64 x 64 tile has little MFMA work per step: a third LDS
+    // stage keeps two steps' copies in flight (4096 x 14336 at M <= 256: 55 -> 34 us).
+    // With more workgroups per CU the LDS is better spent on residency.
+    const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+    return tiles <= 512 ? launch_tile<64, 64, 2, 2, 3>(g, s) : launch_tile<64, 64, 2, 2, 2>(g, s);
+  }
   return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_gemm: no kernel for tile %dx%d", bm, bn);
 }
