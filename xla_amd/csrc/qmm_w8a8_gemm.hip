@@ -531,7 +531,11 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
     return rc;
   }
   if (bm == 128 && bn == 256) return launch_tile<128, 256, 2, 4>(g, s);  // 8 waves, wave tile 64 x 64
-  if (bm == 128 && bn == 128) return launch_tile<128, 128, 2, 2>(g, s);
+  if (bm == 128 && bn == 128) {
+    // one workgroup per CU at most: LDS is free for a third stage (two fit a CU with two stages)
+    const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+    return tiles <= 256 ? launch_tile<128, 128, 2, 2, 3>(g, s) : launch_tile<128, 128, 2, 2, 2>(g, s);
+  }
   if (bm == 64 && bn == 64) {
     // Up to two workgroups per CU there is little else on a CU to cover the latency of a
     // K step's copies with, and a 64 x 64 tile has little MFMA work per step: a third LDS
