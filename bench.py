@@ -51,8 +51,8 @@ def main():
                   help="also run a plain 256 MiB device copy (known traffic, for scaling rocprof byte counters)")
   args = ap.parse_args()
   if args.gpus != 1:
-    print("bench.py: this build measures one GPU; --gpus must be 1 (the kernels are not sharded, "
-          "see DESIGN.md for how the path would shard)", file=sys.stderr)
+    print("bench.py: this build measures one GPU; --gpus must be 1 (the kernels are not sharded: a "
+          "tensor-parallel run would give each GPU its own slice of the output channels)", file=sys.stderr)
     sys.exit(2)
 
   import torch

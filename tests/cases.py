@@ -52,7 +52,7 @@ def rel_l2(a, b):
 
 
 def within_tolerance(actual, expected):
-  """BASELINE tolerance: max-abs-err <= 1e-2 * ||row||_inf for every row, or rel-L2 <= 2e-3."""
+  """Output tolerance of the floating-point paths: max-abs-err <= 1e-2 * ||row||_inf for every row, or rel-L2 <= 2e-3."""
   a, e = actual.double(), expected.double()
   row_ok = ((a - e).abs().amax(-1) <= 1e-2 * e.abs().amax(-1)).all().item()
   return row_ok or rel_l2(a, e) <= 2e-3
