@@ -342,10 +342,11 @@ def test_w8a8_tiles_and_tails(ops):
 
 
 def test_w8a8_pipeline_depths_and_k_steps(ops):
-  # 64 x 64 tiles run with three LDS stages up to 512 tiles and with two above; K from less than one
-  # step (128) to several, with and without a partial last step, crosses every prologue/drain case
-  for (m, n) in ((70, 130), (64 * 24, 64 * 24)):  # 6 tiles, 576 tiles
-    for k in (16, 112, 128, 144, 256, 272, 384, 400, 1040):
+  # 64 x 64 tiles run with three LDS stages up to 512 tiles and with two above, and with two K groups per
+  # workgroup up to 256 tiles when K >= 1024; K from less than one step (128) to several, with and without a
+  # partial last step, even and odd step counts, crosses every prologue/drain case
+  for (m, n) in ((70, 130), (64 * 24, 64 * 24), (64 * 20, 64 * 20)):  # 6 tiles, 576 tiles, 400 tiles
+    for k in (16, 112, 128, 144, 256, 272, 384, 400, 1024, 1040, 1152, 1296):
       g = cases.gen(m + k)
       xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
       w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)

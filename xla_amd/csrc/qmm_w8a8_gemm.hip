@@ -54,21 +54,27 @@ constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 
 // NS = LDS pipeline stages: the copies of NS - 1 K steps are in flight while one is
 // computed.
-template <int BM, int BN, int WM, int WN, int EPI, int NS>
-__global__ void __launch_bounds__(WM * WN * 64)
+// KG = K groups: the workgroup holds KG sets of WM x WN waves; set kg runs the whole
+// pipeline (its own LDS stages) over the K steps kg, kg + KG, ..., and the sets' int32
+// accumulators are added through LDS before the epilogue (exact in any order).  For
+// launches with at most one small tile per CU, whose time is the length of the K loop.
+template <int BM, int BN, int WM, int WN, int EPI, int NS, int KG>
+__global__ void __launch_bounds__(KG * WM * WN * 64)
 qmm_w8a8_gemm_kernel(GemmArgs g) {
-  constexpr int T = WM * WN * 64;
+  constexpr int T = WM * WN * 64;  // threads of one K group
   constexpr int TM = BM / WM, TN = BN / WN;  // wave tile
   constexpr int MI = TM / 32, NI = TN / 32;  // 32x32 MFMA tiles per wave
   constexpr int A_CH = BM * 8 / T, B_CH = BN * 8 / T;  // 16-byte chunks per thread per stage
   static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be a multiple of 32");
   static_assert((BM * 8) % T == 0 && (BN * 8) % T == 0, "tile rows must divide over the threads");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* sA = smem;                      // [NS][BM][128]
-  char* sB = smem + NS * BM * kBK;      // [NS][BN][128]
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps LDS bases in scalar registers
+  // wave-uniform values through readfirstlane: keeps LDS bases in scalar registers
+  const int wave_all = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  const int kg = KG > 1 ? wave_all / (WM * WN) : 0;  // K group of this wave
+  const int wave = wave_all - kg * (WM * WN);         // wave, thread within the group
+  const int tid = (int)threadIdx.x - kg * T, lane = tid & 63;
+  char* sA = smem + kg * (NS * (BM + BN) * kBK);  // [NS][BM][128]
+  char* sB = sA + NS * BM * kBK;                  // [NS][BN][128]
   const int wm = wave / WN, wn = wave % WN;
 
   // Workgroup -> tile.  Consecutive workgroup ids go to different XCDs (8 of
@@ -225,16 +231,23 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   // wave has left at the barrier of step kt.  When step kt is waited for, the steps
   // issued after it are kt+1 .. min(kt + NS - 2, last): they are NS - 2 full stages
   // unless they include the last step, which may be partial (fewer copies per wave).
-  const int ksteps = (K + kBK - 1) / kBK;
+  // With K groups, "step kt" below is the group's own kt-th step, global step
+  // kt * KG + kg; every wave of the workgroup runs the same number of iterations (and
+  // barriers), a group that has run out of steps just meets the others.
+  const int ksteps_all = (K + kBK - 1) / kBK;
+  const int ksteps = (ksteps_all - kg + KG - 1) / KG;   // this group's steps
+  const int kiters = (ksteps_all + KG - 1) / KG;        // iterations of every group
+  auto step_k0 = [&](int kt) { return (kt * KG + kg) * kBK; };
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s)
-    if (s < ksteps) stage_load(s, s * kBK);
+    if (s < ksteps) stage_load(s, step_k0(s));
   int cur = 0, nxt = NS - 1;
-  for (int kt = 0; kt < ksteps; ++kt) {
+  for (int kt = 0; kt < kiters; ++kt) {
     stage_sync(kt + NS - 2 < ksteps - 1);
-    compute(cur, [&]() __attribute__((always_inline)) {
-      if (kt + NS - 1 < ksteps) stage_load(nxt, (kt + NS - 1) * kBK);
-    });
+    if (KG == 1 || kt < ksteps)
+      compute(cur, [&]() __attribute__((always_inline)) {
+        if (kt + NS - 1 < ksteps) stage_load(nxt, step_k0(kt + NS - 1));
+      });
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
@@ -248,20 +261,48 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   static_assert(4 * WM * WN * 32 * kEpStride + 4 * 4 * (BM + BN) <= NS * (BM + BN) * kBK,
                 "epilogue staging must fit in the pipeline's LDS");
   __syncthreads();  // every wave is done reading the last pipeline stage
+  if constexpr (KG > 1) {
+    // Groups 1 .. KG-1 hand their accumulators to group 0, one after the other, through
+    // LDS ([register][thread]: consecutive lanes, consecutive words).  Every wave takes
+    // part in every barrier; the groups other than 0 leave after the last one.
+    static_assert(MI * NI * 16 * T * 4 <= NS * (BM + BN) * kBK, "reduction buffer must fit in one group's stages");
+    int* s_red = (int*)smem + tid;
+    for (int src = 1; src < KG; ++src) {
+      if (kg == src) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_red[((i * NI + j) * 16 + v) * T] = acc[i][j][v];
+      }
+      __syncthreads();
+      if (kg == 0) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] += s_red[((i * NI + j) * 16 + v) * T];
+      }
+      __syncthreads();
+    }
+  }
   float* s_xs = (float*)smem;          // [BM] activation scale
   float* s_xsum = s_xs + BM;           // [BM] round_zpo(float(x_sum))
   float* s_ws = s_xsum + BM;           // [BN] weight scale
   float* s_zp = s_ws + BN;             // [BN] zero point
   int* s_ep = (int*)(s_zp + BN) + wave * (32 * kEpStride);  // per-wave [32][kEpStride]
-  if (tid < BM) {
+  if (kg == 0 && tid < BM) {
     s_xs[tid] = qmm_from_raw(pre_xs, g.x_scale_dt);
     s_xsum[tid] = has_zp ? qmm_round_dt((float)pre_xsum, g.zpo_dt) : 0.f;
   }
-  if (tid < BN) {
+  if (kg == 0 && tid < BN) {
     s_ws[tid] = qmm_from_raw(pre_ws, g.w_scale_dt);
     s_zp[tid] = has_zp ? qmm_from_raw(pre_zp, g.zp_dt) : 0.f;
   }
   __syncthreads();
+  if (KG > 1 && kg != 0) return;  // no barrier below this line
   constexpr int kLanesPerRow = TN / 4;               // each lane finishes 4 consecutive n
   constexpr int kPasses = 32 * kLanesPerRow / 64;    // passes over a 32-row block
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
@@ -384,15 +425,16 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   });
 }
 
-template <int BM, int BN, int WM, int WN, int EPI, int NS>
+template <int BM, int BN, int WM, int WN, int EPI, int NS, int KG>
 int launch_tile_epi(GemmArgs g, hipStream_t stream) {
   g.tiles_m = (g.M + BM - 1) / BM;
   g.tiles_n = (g.N + BN - 1) / BN;
   const int ntiles = g.tiles_m * g.tiles_n;
   const int per = (ntiles + 7) / 8;
   const unsigned grid = (unsigned)(per * 8);
-  constexpr size_t lds = NS * (size_t)(BM + BN) * kBK;
-  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN, EPI, NS>;
+  constexpr size_t lds = KG * NS * (size_t)(BM + BN) * kBK;
+  static_assert(lds <= 160 * 1024 && KG * WM * WN * 64 <= 1024, "workgroup must fit a CU");
+  auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN, EPI, NS, KG>;
   static thread_local bool attr_set = false;
   if (!attr_set) {
     int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
@@ -400,20 +442,20 @@ int launch_tile_epi(GemmArgs g, hipStream_t stream) {
     if (rc != XLA_AMD_QMM_OK) return rc;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WM * WN * 64), lds, stream, g);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(KG * WM * WN * 64), lds, stream, g);
   return QMM_CHECK_LAUNCH("w8a8_gemm launch");
 }
 
 // The short epilogue applies when the scale chain is all f32, there is no zero
 // point, no raw-accumulator output and rows of out are vector-aligned.
-template <int BM, int BN, int WM, int WN, int NS = 2>
+template <int BM, int BN, int WM, int WN, int NS = 2, int KG = 1>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const bool fast = g.out && !g.acc_out && !g.zp && g.cvt_dt == XLA_AMD_DT_F32 &&
                     g.mid_dt == XLA_AMD_DT_F32 && (g.N % 4) == 0 && (g.ldo % 4) == 0 && (((uintptr_t)g.out) & 15) == 0;
-  if (fast && g.out_dt == XLA_AMD_DT_BF16) return launch_tile_epi<BM, BN, WM, WN, 1, NS>(g, stream);
-  if (fast && g.out_dt == XLA_AMD_DT_F16) return launch_tile_epi<BM, BN, WM, WN, 2, NS>(g, stream);
-  if (fast && g.out_dt == XLA_AMD_DT_F32) return launch_tile_epi<BM, BN, WM, WN, 3, NS>(g, stream);
-  return launch_tile_epi<BM, BN, WM, WN, 0, NS>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_BF16) return launch_tile_epi<BM, BN, WM, WN, 1, NS, KG>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_F16) return launch_tile_epi<BM, BN, WM, WN, 2, NS, KG>(g, stream);
+  if (fast && g.out_dt == XLA_AMD_DT_F32) return launch_tile_epi<BM, BN, WM, WN, 3, NS, KG>(g, stream);
+  return launch_tile_epi<BM, BN, WM, WN, 0, NS, KG>(g, stream);
 }
 
 }  // namespace
@@ -541,7 +583,9 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
     // K step's copies with, and a 64 x 64 tile has little MFMA work per step: a third LDS
     // stage keeps two steps' copies in flight (4096 x 14336 at M <= 256: 55 -> 34 us).
     // With more workgroups per CU the LDS is better spent on residency.
+    // At most one workgroup per CU and a long K: two K groups halve the K loop.
     const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
+    if (tiles <= 256 && K >= 1024) return launch_tile<64, 64, 2, 2, 3, 2>(g, s);
     return tiles <= 512 ? launch_tile<64, 64, 2, 2, 3>(g, s) : launch_tile<64, 64, 2, 2, 2>(g, s);
   }
   return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_gemm: no kernel for tile %dx%d", bm, bn);
