@@ -355,6 +355,17 @@ def test_w8a8_pipeline_depths_and_k_steps(ops):
                                  want_acc=True, block_m=64, block_n=64)
       ref = (xq.double() @ w.double().T).long()  # exact: |sum| < 2^53
       assert torch.equal(acc.cpu().long(), ref), (m, n, k)
+  # the short epilogue (whole tiles, f32 scales, no accumulator output) behind two K groups and behind one
+  for (m, n, k) in ((128, 192, 1152), (128, 192, 896)):
+    g = cases.gen(k)
+    xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
+    w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
+    xs, ws = torch.rand(m, 1, generator=g) + 0.5, torch.rand(n, generator=g) + 0.5
+    expect = ((xq.double() @ w.double().T).float() * ws[None, :]) * xs
+    for odt in (torch.float32, torch.bfloat16, torch.float16):
+      out, _ = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), xs.cuda(), ws.cuda(), None, None, cvt_dtype=torch.float32,
+                                 mid_dtype=torch.float32, out_dtype=odt, block_m=64, block_n=64)
+      assert torch.equal(out.cpu(), expect.to(odt)), (m, n, k, odt)
 
 
 def test_w8a8_column_split_two_tile_widths(ops):
