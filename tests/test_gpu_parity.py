@@ -341,6 +341,25 @@ def test_w8a8_tiles_and_tails(ops):
       assert torch.equal(acc.cpu().long(), ref), (bm, bn, m, n, k)
 
 
+@pytest.mark.parametrize("quantize_activation", [False, True])
+def test_q_linear_module_compile_on_gpu(ops, quantize_activation):
+  # test_quantized_matmul.py:128-143 (test_q_linear_module_dynamo): the compiled module runs the HIP kernels
+  from xla_amd.quantization import quantize_linear
+  torch.manual_seed(0)
+  with torch.no_grad():
+    lin = torch.nn.Linear(512, 256, bias=False)
+    x = torch.randn(3, 512)
+    q = quantize_linear(lin, n_bits=8, quantize_activation=quantize_activation)
+    out_quant = q(x)  # CPU tensors: the eager formulation
+    assert torch.allclose(lin(x), out_quant, atol=0.05)
+    qd = q.cuda()
+    before = dict(ops.counters)
+    torch._dynamo.reset()
+    out_compiled = torch.compile(qd, backend="aot_eager", fullgraph=True)(x.cuda())
+    assert sum(ops.counters.values()) > sum(before.values())  # a HIP kernel ran
+    assert torch.allclose(out_compiled.cpu(), out_quant, atol=4e-3)
+
+
 def test_w8a8_pipeline_depths_and_k_steps(ops):
   # 64 x 64 tiles run with three LDS stages up to 512 tiles and with two above, and with two K groups per
   # workgroup up to 256 tiles when K >= 1024; K from less than one step (128) to several, with and without a

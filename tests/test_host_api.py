@@ -175,6 +175,36 @@ def test_rtn_quantizer_and_module_swap(qmm):
   assert torch.allclose(net(x), ref, atol=0.05)
 
 
+def _linear_model(n_in, n_out):
+  class M(torch.nn.Module):
+    def __init__(self):
+      super().__init__()
+      self.linear = torch.nn.Linear(n_in, n_out, bias=False)
+
+    def forward(self, x):
+      return self.linear(x)
+  return M()
+
+
+@pytest.mark.parametrize("quantize_activation", [False, True])
+def test_q_linear_module_compile(qmm, quantize_activation):
+  # test_quantized_matmul.py:128-143 (test_q_linear_module_dynamo) with the backends present here: the op has a
+  # Meta implementation, so the module traces as one opaque call, without graph breaks
+  from xla_amd.quantization import replace_linear_with_quantized
+  torch.manual_seed(0)
+  with torch.no_grad():
+    m = _linear_model(5, 8)
+    x = torch.randn(3, 5)
+    out_fp = m(x)
+    replace_linear_with_quantized(m, n_bits=8, quantize_activation=quantize_activation)
+    out_quant = m(x)
+    assert torch.allclose(out_fp, out_quant, atol=0.02)
+    for backend in ("eager", "aot_eager"):
+      torch._dynamo.reset()
+      out_compiled = torch.compile(m, backend=backend, fullgraph=True)(x)
+      assert torch.allclose(out_compiled, out_quant, atol=4e-3), backend
+
+
 def test_tuned_block_table(qmm):
   from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import TUNED_BLOCK_SIZES, get_tuned_block_sizes
   key0 = next(iter(TUNED_BLOCK_SIZES))
