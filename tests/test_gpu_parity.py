@@ -233,6 +233,48 @@ def test_quantized_matmul_int8_op(ops):
     check(out, exp, "quantized_matmul_int8")
 
 
+def _reference_int8_case(dtype, bs, n_in, n_out, seed):
+  """Inputs and float result of _test_quantized_matmul_int8 (test_pallas.py:886-919): symmetric per-channel
+  qparams from determine_qparams, weights through quantized_decomposed.quantize_per_channel, f32 scalar."""
+  import torch.ao.quantization.fx._decomposed  # noqa: F401  (defines quantized_decomposed for CPU tensors)
+  from torch.ao.quantization.utils import determine_qparams
+  g = cases.gen(seed)
+  x = torch.randn(bs, n_in, generator=g).to(dtype)
+  w = torch.randn(n_out, n_in, generator=g).to(dtype)
+  min_val, max_val = torch.aminmax(w, dim=1)
+  scalar, zero_point = determine_qparams(min_val, max_val, -128, 127, dtype=torch.int8, eps=torch.Tensor([1e-5]),
+                                         has_customized_qrange=False, qscheme=torch.per_channel_symmetric)
+  w_int = torch.ops.quantized_decomposed.quantize_per_channel(w, scalar, zero_point, 0, -128, 127, torch.int8)
+  return x, w_int, scalar.to(torch.float32), torch.nn.functional.linear(x, w)
+
+
+def _rel_error(x, q_x):  # test_pallas.py:882-884
+  abs_error = torch.sqrt(torch.mean(torch.square(q_x - x), axis=1))
+  return torch.mean(abs_error) / torch.sqrt(torch.mean(torch.square(x)))
+
+
+@pytest.mark.parametrize("use_compile", [False, True])
+def test_quantized_matmul_int8_wrapper_like_reference(ops, use_compile):
+  # test_pallas.py:951-1026: shapes in the tuned table (dedicated-kernel semantics) and outside it (fallback +
+  # cast to x.dtype), bf16 and f32, called directly and through torch.compile; bar: rel. error < 3e-2 against
+  # the float linear, result in x's dtype
+  from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import TUNED_BLOCK_SIZES
+  fn = torch.ops.xla.quantized_matmul_int8
+  if use_compile:
+    torch._dynamo.reset()
+    fn = torch.compile(lambda x, w_int, scalar, quantize_activation: torch.ops.xla.quantized_matmul_int8(
+        x, w_int, scalar, quantize_activation=quantize_activation), backend="aot_eager")
+  shapes = [(torch.bfloat16, 256, 4096, 4096), (torch.bfloat16, 512, 4096, 1024)]  # (dtype, bs, n_in, n_out): hits
+  assert all(("gfx950", bs, n_out, n_in, "bfloat16", True) in TUNED_BLOCK_SIZES for _, bs, n_in, n_out in shapes)
+  shapes += [(dt, bs, n_in, n_out) for dt in (torch.bfloat16, torch.float32) for bs in (256, 512)
+             for n_in in (256, 512) for n_out in (256, 512)]  # misses
+  for (dt, bs, n_in, n_out) in shapes:
+    x, w_int, scalar, expected = _reference_int8_case(dt, bs, n_in, n_out, seed=bs + n_in + n_out)
+    actual = fn(x.cuda(), w_int.cuda(), scalar.cuda(), quantize_activation=True).cpu()
+    assert actual.shape == expected.shape and actual.dtype == x.dtype
+    assert _rel_error(expected.float(), actual.float()) < 3e-2, (dt, bs, n_in, n_out)
+
+
 # ---- committed golden fixtures through the HIP path ----------------------------------------
 import json
 import os
