@@ -482,6 +482,36 @@ def test_module_and_state_dict_on_gpu(ops):
     assert qd.weight.is_cuda and set(qd.state_dict()) >= {"weight", "weight_scaler"}
 
 
+def _cosine(x, y):  # _calc_cosine_dist, test_quantized_matmul.py:106-109
+  x, y = x.flatten().to(torch.float32), y.flatten().to(torch.float32)
+  return (torch.sum(x * y) / (torch.norm(x) * torch.norm(y))).item()
+
+
+def test_linear_modules_at_the_reference_tests_shapes(ops):
+  # test_quantized_matmul.py:111-126 (per channel), :182-196 (int4), :228-244 (blockwise), :246-267 (asymmetric
+  # per channel, with and without activation quantization), :269-286 (asymmetric blockwise): tiny layers,
+  # quantized output close to the float one, device output equal to the CPU-tensor one
+  from xla_amd.quantization import quantize_linear
+  torch.manual_seed(0)
+  cases_ = [((5, 8), dict(n_bits=8)), ((5, 8), dict(n_bits=8, quantize_activation=True)), ((5, 8), dict(n_bits=4)),
+            ((6, 8), dict(n_bits=8, block_size=2)), ((6, 8), dict(n_bits=4, block_size=2)),
+            ((6, 8), dict(n_bits=4, symmetric=False)), ((6, 8), dict(n_bits=8, symmetric=False)),
+            ((6, 8), dict(n_bits=4, symmetric=False, quantize_activation=True)),
+            ((6, 8), dict(n_bits=8, symmetric=False, quantize_activation=True)),
+            ((6, 8), dict(n_bits=8, block_size=2, symmetric=False))]
+  with torch.no_grad():
+    for (n_in, n_out), kw in cases_:
+      lin = torch.nn.Linear(n_in, n_out, bias=False)
+      x = torch.randn(3, n_in)
+      out_fp = lin(x)
+      q = quantize_linear(lin, **kw)
+      out_quant = q(x)
+      assert _cosine(out_fp, out_quant) > (0.95 if kw["n_bits"] == 4 else 0.99), kw
+      out_dev = q.cuda()(x.cuda()).cpu()
+      assert _cosine(out_dev, out_quant) > 0.99999, kw
+      assert torch.allclose(out_dev, out_quant, atol=2e-3), kw
+
+
 # ---- quantized_decomposed quantize / dequantize on the GPU ------------------------------------------
 
 def test_qdq_ops_match_oracle_and_torch_cpu(ops):
