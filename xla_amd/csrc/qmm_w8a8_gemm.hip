@@ -1,7 +1,7 @@
 // W8A8 GEMM for gfx950: out[m,n] = epilogue( sum_k x_q[m,k] * w[n,k] ), int8
 // operands, int32 accumulation on the matrix cores (v_mfma_i32_32x32x32_i8),
-// both operands K-contiguous, tiles staged through LDS with a two-stage
-// pipeline, scale epilogue fused.
+// both operands K-contiguous, tiles staged through LDS with a pipeline of two
+// or three stages, scale epilogue fused.
 //
 // Tiling.  A workgroup of WM x WN waves owns a BM x BN tile of the output and
 // walks K in steps of kBK = 128 bytes.  Each wave owns (BM/WM) x (BN/WN)
@@ -48,6 +48,7 @@ __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >>
 // accumulator output, partial tiles); 1/2/3 = all-f32 scale chain with bf16 /
 // f16 / f32 output and nothing else, which whole tiles finish with a short
 // branch-free loop (partial tiles of such a launch still take the general code).
+
 // s_waitcnt immediate for "at most n vector-memory operations outstanding" (n < 64),
 // leaving expcnt and lgkmcnt alone
 constexpr int vmcnt_imm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
