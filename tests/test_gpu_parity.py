@@ -371,7 +371,7 @@ def test_tile_weight_layout(ops):
 
 def test_w8a8_tiles_and_tails(ops):
   # every workgroup tile the kernel offers, on shapes with M/N/K tails
-  for bm, bn in ((32, 32), (64, 64), (128, 128), (128, 256), (256, 256)):
+  for bm, bn in ((32, 32), (64, 32), (64, 64), (128, 128), (128, 256), (256, 256)):
     for (m, n, k) in [(bm + 3, 2 * bn + 5, 144), (17, 33, 64), (bm, bn, 4096)]:
       g = cases.gen(bm + m + n)
       xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
@@ -407,18 +407,20 @@ def test_w8a8_pipeline_depths_and_k_steps(ops):
   # workgroup up to 256 tiles when K >= 1024; K from less than one step (128) to several, with and without a
   # partial last step, even and odd step counts, crosses every prologue/drain case
   # (32 x 32 tiles: four K groups of one wave each when K >= 1024: 1, 2, 3 or 4 of them have a last step)
-  for (m, n, blk) in ((70, 130, 64), (64 * 24, 64 * 24, 64), (64 * 20, 64 * 20, 64), (20, 100, 32)):  # 6, 576, 400, 4 tiles
+  for (m, n, blk, bn) in ((70, 130, 64, 64), (64 * 24, 64 * 24, 64, 64), (64 * 20, 64 * 20, 64, 64), (20, 100, 32, 32),
+                          (70, 100, 64, 32)):  # 6, 576, 400, 4, 8 tiles
     for k in (16, 112, 128, 144, 256, 272, 384, 400, 1024, 1040, 1152, 1296, 1408, 1536):
       g = cases.gen(m + k)
       xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
       w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
       _, acc = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), torch.ones(m, 1).cuda(), torch.ones(n).cuda(), None, None,
                                  cvt_dtype=torch.float32, mid_dtype=torch.float32, out_dtype=torch.float32,
-                                 want_acc=True, block_m=blk, block_n=blk)
+                                 want_acc=True, block_m=blk, block_n=bn)
       ref = (xq.double() @ w.double().T).long()  # exact: |sum| < 2^53
       assert torch.equal(acc.cpu().long(), ref), (m, n, k)
   # the short epilogue (whole tiles, f32 scales, no accumulator output) behind two K groups and behind one
-  for (m, n, k, blk) in ((128, 192, 1152, 64), (128, 192, 896, 64), (32, 96, 1152, 32), (32, 96, 896, 32)):
+  for (m, n, k, blk, bn) in ((128, 192, 1152, 64, 64), (128, 192, 896, 64, 64), (32, 96, 1152, 32, 32), (32, 96, 896, 32, 32),
+                             (128, 96, 1152, 64, 32), (128, 96, 896, 64, 32)):
     g = cases.gen(k)
     xq = torch.randint(-128, 128, (m, k), generator=g, dtype=torch.int32).to(torch.int8)
     w = torch.randint(-128, 128, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
@@ -426,8 +428,8 @@ def test_w8a8_pipeline_depths_and_k_steps(ops):
     expect = ((xq.double() @ w.double().T).float() * ws[None, :]) * xs
     for odt in (torch.float32, torch.bfloat16, torch.float16):
       out, _ = ops.w8a8_gemm_gpu(xq.cuda(), w.cuda(), xs.cuda(), ws.cuda(), None, None, cvt_dtype=torch.float32,
-                                 mid_dtype=torch.float32, out_dtype=odt, block_m=blk, block_n=blk)
-      assert torch.equal(out.cpu(), expect.to(odt)), (m, n, k, blk, odt)
+                                 mid_dtype=torch.float32, out_dtype=odt, block_m=blk, block_n=bn)
+      assert torch.equal(out.cpu(), expect.to(odt)), (m, n, k, blk, bn, odt)
 
 
 def test_w8a8_column_split_two_tile_widths(ops):

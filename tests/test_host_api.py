@@ -57,11 +57,14 @@ def test_dispatcher_regimes():
   tile = (ctypes.c_int32 * 3)()
   assert lib.xla_amd_qmm_w8a8_tile(2048, 14336, 4096, tile) == 0
   assert list(tile) == [256, 256, 128]
-  assert lib.xla_amd_qmm_w8a8_tile(64, 64, 64, tile) == 0 and list(tile)[:2] == [64, 64]
+  assert lib.xla_amd_qmm_w8a8_tile(64, 64, 64, tile) == 0 and list(tile)[:2] == [64, 32]  # few tiles: narrow ones
+  assert lib.xla_amd_qmm_w8a8_tile(32, 4096, 14336, tile) == 0 and list(tile)[:2] == [32, 32]
+  assert lib.xla_amd_qmm_w8a8_tile(128, 14336, 4096, tile) == 0 and list(tile)[:2] == [64, 64]
   # the shape-based choice agrees with the measured best of the tuning sweep on the Llama-3-8B prefill shapes
   from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import TUNED_BLOCK_SIZES
   for (m, n, k) in [(2048, 6144, 4096), (2048, 4096, 4096), (1024, 4096, 4096), (512, 4096, 4096), (512, 14336, 4096),
-                    (4096, 4096, 14336), (2048, 4096, 14336), (256, 28672, 4096), (8192, 1024, 4096)]:
+                    (4096, 4096, 14336), (2048, 4096, 14336), (256, 28672, 4096), (8192, 1024, 4096), (32, 4096, 14336),
+                    (64, 4096, 4096), (128, 4096, 14336), (512, 1024, 4096), (128, 6144, 4096)]:
     assert lib.xla_amd_qmm_w8a8_tile(m, n, k, tile) == 0
     assert tuple(tile) == TUNED_BLOCK_SIZES[("gfx950", m, n, k, "bfloat16", True)], (m, n, k)
 

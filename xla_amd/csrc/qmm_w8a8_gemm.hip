@@ -497,10 +497,11 @@ static double best_column_split(int64_t M, int64_t N, int64_t K, int64_t* n1_out
 // problems take the tile class with the least estimated time.
 static void choose_tile(int64_t M, int64_t N, int64_t K, int* bm, int* bn) {
   auto tiles = [&](int a, int b) { return ((M + a - 1) / a) * ((N + b - 1) / b); };
-  // Decode-sized M with few output columns: 64 x 64 tiles would leave most CUs without
-  // work and fetch 64 activation rows per tile; such a launch is bound by what one CU can
-  // copy from global memory, so spread it over 32 x 32 tiles (four K groups each).
-  if (M <= 32 && tiles(64, 64) <= 128) { *bm = 32; *bn = 32; return; }
+  // Few output tiles: 64 x 64 tiles would leave half of the CUs or more without work.  Such
+  // a launch is bound by what one CU can copy from global memory, so spread it over twice
+  // the tiles, each with four K groups: 32 x 32 for decode-sized M (half the activation rows
+  // fetched per tile as well), else 64 x 32.
+  if (tiles(64, 64) <= 128) { *bm = M <= 32 ? 32 : 64; *bn = 32; return; }
   if (M <= 64 || tiles(64, 64) < 1024) { *bm = 64; *bn = 64; return; }
   int64_t n1;
   const double c256 = M > 128 && N > 128 ? best_column_split(M, N, K, &n1) : 1e30;
@@ -592,6 +593,9 @@ extern "C" int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const v
     const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
     if (tiles <= 256 && K >= 1024) return launch_tile<64, 64, 2, 2, 3, 2>(g, s);
     return tiles <= 512 ? launch_tile<64, 64, 2, 2, 3>(g, s) : launch_tile<64, 64, 2, 2, 2>(g, s);
+  }
+  if (bm == 64 && bn == 32) {  // two waves per K group
+    return K >= 1024 ? launch_tile<64, 32, 2, 1, 3, 4>(g, s) : launch_tile<64, 32, 2, 1, 3, 1>(g, s);
   }
   if (bm == 32 && bn == 32) {
     // one wave per K group; with a short K the groups are not worth their reduction
