@@ -64,7 +64,8 @@ def test_dispatcher_regimes():
   from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import TUNED_BLOCK_SIZES
   for (m, n, k) in [(2048, 6144, 4096), (2048, 4096, 4096), (1024, 4096, 4096), (512, 4096, 4096), (512, 14336, 4096),
                     (4096, 4096, 14336), (2048, 4096, 14336), (256, 28672, 4096), (8192, 1024, 4096), (32, 4096, 14336),
-                    (64, 4096, 4096), (128, 4096, 14336), (512, 1024, 4096), (128, 6144, 4096)]:
+                    (64, 4096, 4096), (128, 4096, 14336), (512, 1024, 4096), (128, 6144, 4096), (256, 14336, 4096),
+                    (128, 28672, 4096), (512, 6144, 4096)]:
     assert lib.xla_amd_qmm_w8a8_tile(m, n, k, tile) == 0
     assert tuple(tile) == TUNED_BLOCK_SIZES[("gfx950", m, n, k, "bfloat16", True)], (m, n, k)
 

@@ -492,8 +492,9 @@ static double best_column_split(int64_t M, int64_t N, int64_t K, int64_t* n1_out
 }
 
 // Tile choice by shape: 64 x 64 tiles (several workgroups resident per CU, which hides
-// the latency of their short K steps) while there are fewer than four per CU: measured
-// faster than one round of 128 x 128 tiles up to there, for K = 2048 ... 14336.  Larger
+// the latency of their short K steps) while there are at most three per CU: measured
+// faster than one round of 128 x 128 tiles up to there, for K = 2048 ... 14336 (at 208 to 256
+// tiles of 128 x 128, three stages, the larger tile is 8 % faster).  Larger
 // problems take the tile class with the least estimated time.
 static void choose_tile(int64_t M, int64_t N, int64_t K, int* bm, int* bn) {
   auto tiles = [&](int a, int b) { return ((M + a - 1) / a) * ((N + b - 1) / b); };
@@ -502,7 +503,7 @@ static void choose_tile(int64_t M, int64_t N, int64_t K, int* bm, int* bn) {
   // the tiles, each with four K groups: 32 x 32 for decode-sized M (half the activation rows
   // fetched per tile as well), else 64 x 32.
   if (tiles(64, 64) <= 128) { *bm = M <= 32 ? 32 : 64; *bn = 32; return; }
-  if (M <= 64 || tiles(64, 64) < 1024) { *bm = 64; *bn = 64; return; }
+  if (M <= 64 || tiles(64, 64) <= 768) { *bm = 64; *bn = 64; return; }
   int64_t n1;
   const double c256 = M > 128 && N > 128 ? best_column_split(M, N, K, &n1) : 1e30;
   const double c128x256 = N > 128 ? kLaunchUs + rounds_us(kCost128x256, tiles(128, 256), K) : 1e30;

@@ -32,13 +32,13 @@ _MEASURED = {
                    2048: (128, 256), 4096: (256, 256), 8192: (256, 256)},
     (1024, 4096): {32: (32, 32), 64: (64, 32), 128: (64, 32), 256: (64, 32), 512: (64, 32), 1024: (64, 64),
                    2048: (64, 64), 4096: (64, 64), 8192: (128, 256)},
-    (14336, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (64, 64), 512: (128, 256), 1024: (256, 256),
+    (14336, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (128, 128), 512: (128, 256), 1024: (256, 256),
                     2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
     (4096, 14336): {32: (32, 32), 64: (64, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64), 1024: (128, 128),
                     2048: (128, 256), 4096: (256, 256), 8192: (256, 256)},
     (6144, 4096): {32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (128, 256),
                    2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
-    (28672, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (128, 256), 512: (256, 256), 1024: (256, 256),
+    (28672, 4096): {32: (64, 64), 64: (64, 64), 128: (128, 128), 256: (128, 256), 512: (256, 256), 1024: (256, 256),
                     2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
     (8192, 8192): {32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128), 1024: (128, 256),
                    2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
