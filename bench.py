@@ -251,6 +251,17 @@ def main():
       _, ev, _ = time_calls([run_fused], 20, 5, use_graph)
       extra[f"llama3_8b_layer_linears_{tag}"]["us_qkv_and_gate_up_fused"] = round(ev * 1e3, 2)
       del fused_s
+    # W8A8 GEMM with few output tiles: the down projection (4096 x 14336) at decode-sized M
+    wd, sd = layer["down"]
+    small = {}
+    for m in (32, 128, 512):
+      xq_s, xs_s, _ = qmm.quantize_per_token_gpu(torch.randn(m, 14336, generator=g5).bfloat16().to(dev))
+      _, ev, _ = time_calls([lambda: qmm.w8a8_gemm_gpu(xq_s, wd, xs_s, sd, None, None, cvt_dtype=torch.float32,
+                                                       mid_dtype=torch.float32, out_dtype=torch.bfloat16)],
+                            20, 5, use_graph)
+      small[f"M{m}_us"] = round(ev * 1e3, 2)
+    small["note"] = "GEMM alone, bf16 output, weights (59 MB) cache-warm; M=32: 32x32 tiles, M=128: 64x32, M=512: 64x64"
+    extra["w8a8_gemm_4096x14336_small_M"] = small
     # quantized_decomposed quantize / dequantize of a weight-sized tensor (HBM-bound elementwise)
     import xla_amd.experimental.quantized  # noqa: F401
     qd = torch.ops.quantized_decomposed
