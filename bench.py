@@ -70,7 +70,15 @@ def main():
   op = torch.ops.xla.quantized_matmul
 
   def time_calls(fns, steps, warmup, graph=True):
-    """fns: list of zero-arg callables used round-robin.  Returns (wall_ms_per_step, event_ms_per_step)."""
+    """fns: list of zero-arg callables used round-robin.  Returns (wall_ms_per_step, event_ms_per_step, graphed).
+
+    Every callable runs once before the warm-up, whatever `warmup` is: one-time work of a first
+    call (the tiled copy of a weight) must be done before anything is captured or timed, and the
+    count of such re-layouts is checked not to move afterwards."""
+    for f in fns:
+      f()
+    torch.cuda.synchronize()
+    relayouts = qmm.counters["pack"]
     for i in range(warmup):
       fns[i % len(fns)]()
     torch.cuda.synchronize()
@@ -98,6 +106,7 @@ def main():
     e1.record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    assert qmm.counters["pack"] == relayouts, "a weight was re-laid out inside the captured / timed region"
     return (t1 - t0) * 1e3 / steps, e0.elapsed_time(e1) / steps, g is not None
 
   use_graph = not args.no_graph

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define XLA_AMD_QMM_ABI_VERSION 2
+#define XLA_AMD_QMM_ABI_VERSION 3
 
 /* return codes */
 #define XLA_AMD_QMM_OK 0
@@ -44,15 +44,15 @@ extern "C" {
 #define XLA_AMD_DT_BF16 1
 #define XLA_AMD_DT_F16 2
 
-/* float -> int8 conversion of a rounded value outside [-128,127]
- * (reference: `.to(torch.int8)` with no clamp, xla_quantized_matmul.py:72;
- * XLA's ConvertElementType saturates, torch's CPU cast wraps modulo 256). */
 /* integer dtypes of quantized tensors (quantize_affine / dequantize_affine) */
 #define XLA_AMD_QDT_I8 0
 #define XLA_AMD_QDT_U8 1
 #define XLA_AMD_QDT_I16 2
 #define XLA_AMD_QDT_I32 3
 
+/* float -> int8 conversion of a rounded value outside [-128,127]
+ * (reference: `.to(torch.int8)` with no clamp, xla_quantized_matmul.py:72;
+ * XLA's ConvertElementType saturates, torch's CPU cast wraps modulo 256). */
 #define XLA_AMD_OVERFLOW_SATURATE 0
 #define XLA_AMD_OVERFLOW_WRAP 1
 
@@ -119,6 +119,15 @@ int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, 
                             int src_layout, int bits, void* stream);
 
 /*
+ * Inverse of xla_amd_qmm_tile_weight: rebuilds the operator's int8 container
+ * ([N, K] for XLA_AMD_W_NK, [S, C, N] for XLA_AMD_W_SCN) from a tiled copy, so
+ * that a module which keeps only the tiled form on the device can still save
+ * the reference's `weight` buffer (xla_quantized_matmul.py:202, :231) unchanged.
+ */
+int xla_amd_qmm_untile_weight(const void* tiled, int8_t* w, int64_t S, int64_t C, int64_t N,
+                              int dst_layout, int bits, void* stream);
+
+/*
  * Weight-only quantized matmul, fast path: streams a tiled weight once and
  * keeps up to 32 rows of x per pass in MFMA fragments (passes over w repeat
  * for larger M).  Replaces, with the reference's rounding points,
@@ -131,11 +140,19 @@ int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, 
  * and scale / zp of x's dtype (the reference's einsum raises on mixed dtypes);
  * else XLA_AMD_QMM_EUNSUPPORTED.
  * out_dt must be the torch promotion of (x_dt, scale_dt).
+ * dot_dt is the dtype the dot product is rounded to before it is scaled: x_dt
+ * for quantized_matmul (the XLA dot's result has x's type, csrc/ops/ops.cpp:252-259),
+ * or XLA_AMD_DT_F32 (per-channel only) for the float branch of the Pallas kernel,
+ * which keeps a float32 accumulator, scales it and casts once
+ * (pallas_kernels/quantized_matmul_kernel.py:108-121, :246).
+ * store_dt is the dtype out is stored as: out_dt, or the type of a final cast
+ * of the result (`.to(x.dtype)`, custom_kernel.py:1105-1106; `.astype`,
+ * quantized_matmul_kernel.py:121).
  */
 int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const void* scale,
                                    const void* zp, void* out, int64_t M, int64_t N, int64_t K,
                                    int64_t C, int bits, int x_dt, int scale_dt, int zp_dt,
-                                   int out_dt, void* stream);
+                                   int dot_dt, int out_dt, int store_dt, void* stream);
 
 /*
  * Weight-only quantized matmul for any shape, reading the operator's own
@@ -146,7 +163,7 @@ int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const voi
 int xla_amd_qmm_weight_only_generic(const void* x, const int8_t* w, const void* scale,
                                     const void* zp, void* out, int64_t M, int64_t N, int64_t K,
                                     int64_t C, int w_layout, int x_dt, int scale_dt, int zp_dt,
-                                    int out_dt, void* stream);
+                                    int dot_dt, int out_dt, int store_dt, void* stream);
 
 /*
  * Per-token dynamic activation quantization (`_quantize_tensor`,
@@ -156,7 +173,8 @@ int xla_amd_qmm_weight_only_generic(const void* x, const int8_t* w, const void* 
  * with every intermediate rounded to x_dt as the reference does op by op.
  * x [M,K], x_q int8 [M,K], x_scale [M] stored as scale_out_dt (x_dt for the
  * torch op, f32 for the Pallas variant).  A row of zeros yields x_q = 0,
- * scale = 0 (the reference leaves this case undefined).
+ * scale = 0; a row that holds a NaN yields scale = NaN (as torch.amax does)
+ * and x_q = 0 (the reference leaves both cases undefined).
  * x_sum (nullable) receives sum_k x_q[m,k] as int32 [M]: the factor of the
  * zero-point term once x has been replaced by its quantized form (:109,:128).
  */
@@ -193,6 +211,32 @@ int xla_amd_qmm_w8a8_gemm(const int8_t* x_q, const int8_t* w, const void* x_scal
                           int32_t* acc_out, int64_t M, int64_t N, int64_t K, int x_scale_dt,
                           int w_scale_dt, int zp_dt, int cvt_dt, int mid_dt, int zpo_dt,
                           int out_dt, int block_m, int block_n, void* stream);
+
+/*
+ * Bytes of workspace xla_amd_qmm_w8a8_linear needs for an [M, K] activation
+ * against an [N, K] weight (0 for arguments it rejects).
+ */
+size_t xla_amd_qmm_w8a8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * The whole `quantize_activation=True` operator in one call: the statements of
+ * xla_amd_qmm_quantize_per_token followed by those of xla_amd_qmm_w8a8_gemm
+ * (xla_quantized_matmul.py:108-114, :125-135; Pallas wrapper
+ * pallas_kernels/quantized_matmul_kernel.py:199-221 with its matmul_kernel).
+ * x [M,K] of x_dt, w int8 [N,K], w_scale [N], zp [N] or NULL, out [M,N].
+ * The quantized activations (int8 [M,K]), their scales (stored as x_scale_dt:
+ * x_dt for the torch operator, f32 for the Pallas variant) and, with a zero
+ * point, their row sums live in `workspace`: device memory of at least
+ * xla_amd_qmm_w8a8_linear_workspace_bytes(M, N, K) bytes, 256-byte aligned,
+ * which the call may overwrite entirely and does not need afterwards.
+ * cvt_dt / mid_dt / out_dt, block_m / block_n as for xla_amd_qmm_w8a8_gemm
+ * (the zero-point term is rounded to zp_dt).
+ */
+int xla_amd_qmm_w8a8_linear(const void* x, const int8_t* w, const void* w_scale, const void* zp,
+                            void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                            int64_t K, int x_dt, int w_scale_dt, int zp_dt, int x_scale_dt, int cvt_dt,
+                            int mid_dt, int out_dt, int overflow_policy, int block_m, int block_n,
+                            void* stream);
 
 /*
  * Shape-based choice between the kernels (the role of the tuned-table lookup

@@ -30,11 +30,21 @@ How each function is pinned (tests/test_oracle_*.py):
                          matmul on dequantized weights within the reference's
                          thresholds, and the committed tests/golden fixtures.
   quantized_matmul_int8  same integer model + f32 epilogue closed form; the
-                         reference pins it only on TPU within rel-err 2e-2.
+                         float branch (quantize_activation=False) against
+                         bf16(f64 dot * scale) within one ulp, w == 1 (row sums)
+                         and one-hot x; the reference pins the kernel only on
+                         TPU, only with quantize_activation=True, within
+                         rel-err 2e-2.
 Parity unpinned (cannot be decided offline, see the policy argument):
   float->int8 conversion of a rounded value of +-128 on the PJRT CPU device
   (`overflow`), and whether XLA-CPU keeps bf16 round trips between the
   elementwise ops of the quantizer.
+  quantized_matmul_int8(quantize_activation=False) with bf16/f16 x: the Pallas
+  kernel calls lax.dot_general on (x, int8 w) without preferred_element_type
+  (quantized_matmul_kernel.py:108-112); whether each in-block dot comes back in
+  float32 or rounded to x's dtype is decided by jax 0.8.0.dev20251001 / Mosaic,
+  which are not part of the reference tree.  This restatement keeps the float32
+  accumulator the kernel declares (acc_dtype, :246) over all of K.
 """
 import torch
 import torch.nn.functional as F
@@ -64,7 +74,7 @@ def quantize_tensor(x: torch.Tensor, n_bits: int = 8, dim: int = -1, overflow: s
   scale = max_val / int_max
   r = torch.round(x / scale)
   x_int = _to_int8(r, overflow)
-  scale = torch.nan_to_num(scale, nan=0.0)
+  # (an all-zero row gives scale 0 and quotients 0/0 -> 0; a row that holds a NaN keeps its NaN scale)
   return x_int, scale.to(x.dtype)
 
 
@@ -109,7 +119,7 @@ def pallas_quantize_array(x: torch.Tensor, overflow: str = "saturate"):
   scale = x_abs_max / 127
   r = torch.round(x / scale)
   x_int = _to_int8(r, overflow)
-  return x_int, torch.nan_to_num(scale, nan=0.0).to(torch.float32)
+  return x_int, scale.to(torch.float32)
 
 
 def quantized_matmul_int8(x, w, scalar, quantize_activation=False, overflow="saturate"):

@@ -1,0 +1,333 @@
+"""GPU parity at the full benchmark shapes of a decoder layer, the dedicated int8 operator at the full prefill
+shape, the float branch of the dedicated kernel, and the device-side weight layout of the module."""
+import numpy as np
+import pytest
+import torch
+
+from tests import cases
+from oracle import quantized_matmul_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+# the seven linears of one Llama-3-8B decoder layer: name -> (out features, in features)
+LAYER = {"q": (4096, 4096), "k": (1024, 4096), "v": (1024, 4096), "o": (4096, 4096),
+         "gate": (14336, 4096), "up": (14336, 4096), "down": (4096, 14336)}
+
+
+@pytest.fixture(scope="module")
+def ops():
+  import xla_amd.experimental.custom_kernel  # noqa: F401  (defines both ops)
+  import xla_amd.experimental.xla_quantized_matmul as qmm
+  return qmm
+
+
+@pytest.fixture(scope="module")
+def layer():
+  """name -> (w int8 [out, in], scale f32 [out]) for every linear, seeded."""
+  out = {}
+  for i, (name, (n, k)) in enumerate(LAYER.items()):
+    _, w, s, _ = cases.per_channel_int8(1, n, k, torch.bfloat16, torch.float32, seed=100 + i)
+    out[name] = (w, s)
+  return out
+
+
+def check(actual, expected, what=""):
+  assert actual.dtype == expected.dtype, f"{what}: dtype {actual.dtype} vs {expected.dtype}"
+  assert actual.shape == expected.shape
+  a = actual.cpu()
+  assert torch.isfinite(a.float()).all()
+  rl2 = cases.rel_l2(a, expected)
+  assert cases.within_tolerance(a, expected), f"{what}: rel-L2 {rl2:.3e} outside tolerance"
+  return rl2
+
+
+def exact_acc(xq, w):
+  """int8 x int8 -> exact integer contraction through float64 BLAS (|sum| < 2^53)."""
+  return (xq.double() @ w.double().T).long()
+
+
+# ---- config 5, decode step: x bf16 [32, in] through the streaming kernel --------------------------------
+@pytest.mark.parametrize("name", list(LAYER))
+def test_config5_decode_m32(ops, layer, name):
+  w, s = layer[name]
+  n, k = LAYER[name]
+  x = torch.randn(32, k, generator=cases.gen(7)).bfloat16()
+  s16 = s.bfloat16()
+  exp = oracle.quantized_matmul(x, w, s16)
+  before = ops.counters["skinny_mfma"]
+  out = torch.ops.xla.quantized_matmul(x.cuda(), w.cuda(), s16.cuda())
+  assert ops.counters["skinny_mfma"] == before + 1
+  rl2 = check(out, exp, f"cfg5 decode {name}")
+  assert rl2 < 5e-4, rl2
+
+
+# ---- config 5, prefill chunk: x bf16 [512, in] through W8A8 ----------------------------------------------
+@pytest.mark.parametrize("name", list(LAYER))
+def test_config5_prefill_m512(ops, layer, name):
+  w, s = layer[name]
+  n, k = LAYER[name]
+  x = cases.outlier_activations(512, k, torch.bfloat16, seed=11)
+  xd, wd, sd = x.cuda(), w.cuda(), s.cuda()
+  # quantizer: bit exact
+  xq_ref, xs_ref = oracle.quantize_tensor(x)
+  xq, xs, _ = ops.quantize_per_token_gpu(xd)
+  assert torch.equal(xq.cpu(), xq_ref) and torch.equal(xs.cpu(), xs_ref)
+  # int32 accumulators: bit exact over the whole output (K = 14336: |acc| up to 233 M)
+  acc_ref = exact_acc(xq_ref, w)
+  assert acc_ref.abs().max() < 2**31
+  _, acc = ops.w8a8_gemm_gpu(xq, wd, xs, sd, None, None, cvt_dtype=torch.float32, mid_dtype=torch.float32,
+                             out_dtype=torch.float32, want_acc=True)
+  assert torch.equal(acc.cpu().long(), acc_ref), f"cfg5 prefill {name}: accumulators differ"
+  # the operator: rows against the oracle, everything against the epilogue applied to the exact accumulators
+  before = ops.counters["w8a8_mfma"]
+  out = torch.ops.xla.quantized_matmul(xd, wd, sd, quantize_activation=True)
+  assert ops.counters["w8a8_mfma"] == before + 1
+  assert out.dtype == torch.float32
+  rows = torch.arange(0, 512, 16)
+  check(out[rows.cuda()], oracle.quantized_matmul(x[rows], w, s, quantize_activation=True), f"cfg5 prefill {name}")
+  expect = (acc_ref.float() * s) * xs_ref.float()
+  assert torch.equal(out.cpu(), expect)
+
+
+def test_config5_fused_projections(ops, layer):
+  # q/k/v and gate/up concatenated along N: one launch each, outputs identical to the separate layers
+  from xla_amd.experimental.xla_quantized_matmul import XlaQuantizedLinear
+  from xla_amd.quantization import fuse_quantized_linears
+  for qa, m in ((False, 32), (True, 512)):
+    x = cases.outlier_activations(m, 4096, torch.bfloat16, seed=13).cuda()
+    for names in (("q", "k", "v"), ("gate", "up")):
+      mods = []
+      for nm in names:
+        w, s = layer[nm]
+        lin = XlaQuantizedLinear(4096, w.shape[0], is_symmetric=True, quantize_activation=qa)
+        lin.load_quantized_weight(w.cuda(), (s if qa else s.bfloat16()).cuda())
+        mods.append(lin)
+      fused = fuse_quantized_linears(mods)
+      outs = fused(x).split([l.output_dim for l in mods], dim=-1)
+      for nm, l, o in zip(names, mods, outs):
+        assert torch.equal(l(x), o), (qa, nm)
+      w0, s0 = layer[names[0]]
+      exp = oracle.quantized_matmul(x.cpu()[:8], w0, s0 if qa else s0.bfloat16(), quantize_activation=qa)
+      check(outs[0][:8], exp, f"fused {names} qa={qa}")
+
+
+# ---- config 4 in its "bf16 out" form: the dedicated int8 operator at 2048 x 14336 x 4096 -----------------
+def test_config4_quantized_matmul_int8_bf16_out_full(ops):
+  m, n, k = 2048, 14336, 4096
+  x = cases.outlier_activations(m, k, torch.bfloat16, seed=1234)
+  _, w, s, _ = cases.per_channel_int8(1, n, k, torch.bfloat16, torch.float32, seed=31)
+  from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import TUNED_BLOCK_SIZES
+  assert ("gfx950", m, n, k, "bfloat16", True) in TUNED_BLOCK_SIZES  # table hit: the dedicated kernel
+  out = torch.ops.xla.quantized_matmul_int8(x.cuda(), w.cuda(), s.cuda(), quantize_activation=True)
+  assert out.dtype == torch.bfloat16 and out.shape == (m, n)
+  rows = torch.arange(0, m, 61)
+  check(out[rows.cuda()], oracle.quantized_matmul_int8(x[rows], w, s, quantize_activation=True), "cfg4 bf16 rows")
+  # every element: the kernel's documented chain on exact accumulators (f32 scale of the activations)
+  xq_ref, xs_ref = oracle.pallas_quantize_array(x)
+  expect = ((exact_acc(xq_ref, w).float() * s) * xs_ref).to(torch.bfloat16)
+  assert torch.equal(out.cpu(), expect)
+  # size-independent property: the output is linear in the weight scale (a power of two scales bf16 exactly)
+  out4 = torch.ops.xla.quantized_matmul_int8(x.cuda(), w.cuda(), (s * 4).cuda(), quantize_activation=True)
+  assert torch.equal(out4, out * 4)
+
+
+# ---- the float branch of the dedicated kernel (f32 accumulation, f32 scale, one cast) --------------------
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
+def test_dedicated_kernel_float_branch(ops, xdt):
+  from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import quantized_matmul_int8 as kernel
+  for (m, n, k) in [(16, 14336, 4096), (5, 256, 1024), (40, 100, 384), (3, 8, 5)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)
+    exp = oracle.quantized_matmul_int8(x, w, s, quantize_activation=False)
+    with pytest.raises(AssertionError):
+      kernel(x.cuda(), w.cuda(), s.cuda())  # all three block sizes are required (:194)
+    out = kernel(x.cuda(), w.cuda(), s.cuda(), batch_block_size=128, out_block_size=128, in_block_size=128)
+    assert out.dtype == xdt
+    rl2 = check(out, exp, f"float branch {m, n, k, xdt}")
+    assert rl2 < 3e-4, rl2
+    if xdt == torch.bfloat16 and k >= 1024:
+      # one rounding, not the two of quantized_matmul: closer to the float64 result than that sequence is
+      exact = (x.double() @ w.double().T) * s.float().double()
+      two = torch.ops.xla.quantized_matmul(x.cuda(), w.cuda(), s.cuda()).cpu()
+      assert cases.rel_l2(out.cpu(), exact) < 0.8 * cases.rel_l2(two, exact)
+  # block sizes the GEMM has no tile for are hints only (the reference ignores caller block sizes altogether)
+  x = cases.outlier_activations(256, 512, torch.bfloat16, seed=3)
+  _, w, s, _ = cases.per_channel_int8(1, 384, 512, torch.bfloat16, torch.float32, seed=4)
+  out = kernel(x.cuda(), w.cuda(), s.cuda(), quantize_activation=True, batch_block_size=256, out_block_size=512,
+               in_block_size=512)
+  check(out, oracle.quantized_matmul_int8(x, w, s, quantize_activation=True), "hint block sizes")
+  # the wrapper always takes its block sizes from the table, whatever the caller passes (custom_kernel.py:1088-1091)
+  out = torch.ops.xla.quantized_matmul_int8(x.cuda(), w.cuda(), s.cuda(), None, None, True, 512, 512, 512)
+  check(out, oracle.quantized_matmul_int8_fallback(x, w, s, quantize_activation=True), "wrapper, table miss")
+  # weight-only through the wrapper: never in the table -> the quantized_matmul route, cast to x.dtype
+  x, w, s, _ = cases.per_channel_int8(8, 256, 512, torch.bfloat16, torch.float32, seed=5)
+  out = torch.ops.xla.quantized_matmul_int8(x.cuda(), w.cuda(), s.cuda())
+  assert out.dtype == torch.bfloat16
+  check(out, oracle.quantized_matmul_int8_fallback(x, w, s), "wrapper weight-only")
+
+
+def test_fused_linear_entry_point_matches_two_calls(ops):
+  # xla_amd_qmm_w8a8_linear (quantize + GEMM in one call, activations in a workspace) against the two separate calls
+  for (m, n, k, sdt, zp) in [(200, 384, 512, torch.float32, False), (200, 384, 512, torch.bfloat16, True),
+                             (7, 9, 80, torch.float32, True), (512, 1024, 4096, torch.float32, False)]:
+    x = cases.outlier_activations(m, k, torch.bfloat16, seed=m)
+    _, w, s, _ = cases.per_channel_int8(1, n, k, torch.bfloat16, sdt, seed=n)
+    z = (torch.randn(n, generator=cases.gen(3)) * 0.01).to(sdt) if zp else None
+    xd, wd, sd = x.cuda(), w.cuda(), s.cuda()
+    zd = None if z is None else z.cuda()
+    odt = torch.promote_types(sdt, torch.bfloat16)
+    xq, xs, xsum = ops.quantize_per_token_gpu(xd, want_sum=zp)
+    two, _ = ops.w8a8_gemm_gpu(xq, wd, xs, sd, zd, xsum, cvt_dtype=sdt, mid_dtype=sdt, out_dtype=odt)
+    one = ops.w8a8_linear_gpu(xd, wd, sd, zd, x_scale_dtype=torch.bfloat16, cvt_dtype=sdt, mid_dtype=sdt, out_dtype=odt)
+    assert torch.equal(one, two), (m, n, k, sdt, zp)
+    check(one, oracle.quantized_matmul(x, w, s, z, quantize_activation=True), "fused linear")
+
+
+# ---- device-side weight layout: explicit preparation, invalidation, capture, memory ----------------------
+def test_prepare_release_and_state_dict(ops):
+  from xla_amd.quantization import quantize_linear
+  torch.manual_seed(3)
+  for kw in (dict(n_bits=8, scale_dtype=torch.bfloat16), dict(n_bits=4, block_size=128, symmetric=False,
+                                                              scale_dtype=torch.bfloat16)):
+    lin = torch.nn.Linear(512, 256, bias=False)
+    q = quantize_linear(lin, **kw).cuda()
+    x = torch.randn(5, 512).bfloat16().cuda()
+    ref = q(x)
+    sd_before = {k: v.clone() for k, v in q.state_dict().items()}
+    assert q.prepare() is True
+    packs = ops.counters["pack"]
+    assert torch.equal(q(x), ref)
+    assert ops.counters["pack"] == packs  # the forward used the module's own tiled copy
+    assert q.prepare(release_weight=True) is True
+    assert q.weight.numel() == 0  # the reference-layout buffer is gone from the device ...
+    assert torch.equal(q(x), ref)
+    sd = q.state_dict()  # ... and comes back, unchanged, when the module is saved
+    assert sorted(sd) == sorted(sd_before)
+    for key in sd:
+      assert sd[key].shape == sd_before[key].shape and torch.equal(sd[key], sd_before[key]), key
+    # loading restores the buffer; preparing again releases it again
+    q.load_state_dict(sd)
+    assert q.weight.shape == sd_before["weight"].shape and torch.equal(q(x), ref)
+    q.prepare(release_weight=True)
+    assert torch.equal(q(x), ref)
+    # torch.compile traces the tiled operator as one opaque call
+    torch._dynamo.reset()
+    assert torch.equal(torch.compile(q, backend="aot_eager", fullgraph=True)(x), ref)
+  # layers without a tiled copy: W8A8, shapes of the generic kernel, CPU modules
+  assert quantize_linear(torch.nn.Linear(512, 256, bias=False), quantize_activation=True).cuda().prepare() is False
+  assert quantize_linear(torch.nn.Linear(6, 8, bias=False)).cuda().prepare() is False
+  assert quantize_linear(torch.nn.Linear(512, 256, bias=False)).prepare() is False
+
+
+def test_weight_cache_sees_data_writes_after_invalidate_and_inference_tensors(ops):
+  x, w, s, _ = cases.per_channel_int8(4, 64, 256, torch.bfloat16, torch.bfloat16, seed=1)
+  _, w2, _, _ = cases.per_channel_int8(4, 64, 256, torch.bfloat16, torch.bfloat16, seed=2)
+  xd, wd, sd = x.cuda(), w.cuda(), s.cuda()
+  op = torch.ops.xla.quantized_matmul
+  out1 = op(xd, wd, sd)
+  check(out1, oracle.quantized_matmul(x, w, s), "first weight")
+  wd.copy_(w2.cuda())  # in place through torch: the version counter moves, the copy is remade
+  check(op(xd, wd, sd), oracle.quantized_matmul(x, w2, s), "in-place write")
+  wd.data.copy_(w.cuda())  # bypasses the version counter: needs the explicit invalidation
+  ops.invalidate_weight_cache(wd)
+  check(op(xd, wd, sd), oracle.quantized_matmul(x, w, s), "data write + invalidate")
+  with torch.inference_mode():
+    wi = w2.cuda()  # an inference tensor: no version counter
+    check(op(xd, wi, sd), oracle.quantized_matmul(x, w2, s), "inference-mode weight")
+    check(op(xd, wi, sd), oracle.quantized_matmul(x, w2, s), "inference-mode weight, cached")
+
+
+def test_graph_capture_needs_a_prepared_weight(ops):
+  x, w, s, _ = cases.per_channel_int8(4, 64, 256, torch.bfloat16, torch.bfloat16, seed=5)
+  xd, wd, sd = x.cuda(), w.cuda(), s.cuda()
+  op = torch.ops.xla.quantized_matmul
+  exp = oracle.quantized_matmul(x, w, s)
+  torch.cuda.synchronize()
+  g = torch.cuda.CUDAGraph()
+  with pytest.raises(RuntimeError, match="prepare"):
+    with torch.cuda.graph(g):
+      op(xd, wd, sd)
+  torch.cuda.synchronize()
+  assert ops.prepare_weight(wd) is True
+  static_out = None
+  g = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(g):
+    static_out = op(xd, wd, sd)
+  for _ in range(3):  # every replay, with eager work in between, gives the eager result
+    g.replay()
+    torch.cuda.synchronize()
+    check(static_out, exp, "graph replay")
+    check(op(xd, wd, sd), exp, "eager between replays")
+
+
+def test_quantizer_nan_row(ops):
+  x = cases.outlier_activations(6, 512, torch.bfloat16, seed=2)
+  x[2, 100] = float("nan")
+  x[4] = 0
+  q_ref, s_ref = oracle.quantize_tensor(x)
+  q, s, _ = ops.quantize_per_token_gpu(x.cuda())
+  assert torch.equal(q.cpu(), q_ref)
+  assert torch.isnan(s.cpu()[2]).all() and torch.isnan(s_ref[2]).all()
+  keep = torch.tensor([0, 1, 3, 4, 5])
+  assert torch.equal(s.cpu()[keep], s_ref[keep])
+
+
+def test_qdq_per_channel_single_entry_parameters(ops):
+  # scale with one entry per channel and a single zero point, and the reverse
+  import xla_amd.experimental.quantized  # noqa: F401
+  qd = torch.ops.quantized_decomposed
+  g = cases.gen(8)
+  x = torch.randn(6, 10, 16, generator=g) * 3
+  for axis in (0, 1):
+    c = x.shape[axis]
+    scales = torch.rand(c, generator=g) * 0.1 + 0.01
+    zps = torch.randint(-20, 20, (c,), generator=g)
+    for sc, zp in ((scales, zps[:1]), (scales[:1], zps)):
+      q = qd.quantize_per_channel(x.cuda(), sc.cuda(), zp.cuda(), axis, -128, 127, torch.int8)
+      ref = qd.quantize_per_channel(x, sc.expand(c).contiguous(), zp.expand(c).contiguous(), axis, -128, 127, torch.int8)
+      assert torch.equal(q.cpu(), ref), (axis, sc.numel(), zp.numel())
+      d = qd.dequantize_per_channel(q, sc.cuda(), zp.cuda(), axis, -128, 127, torch.int8)
+      dref = qd.dequantize_per_channel(ref, sc.expand(c).contiguous(), zp.expand(c).contiguous(), axis, -128, 127, torch.int8)
+      assert torch.equal(d.cpu(), dref)
+  # second call with the same parameter tensors: checked already, no host round trip, capturable
+  sc, zp = scales.cuda(), zps.cuda()
+  xd = x.cuda()
+  first = qd.quantize_per_channel(xd, sc, zp, 1, -128, 127, torch.int8)
+  torch.cuda.synchronize()
+  gr = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(gr):
+    again = qd.quantize_per_channel(xd, sc, zp, 1, -128, 127, torch.int8)
+  gr.replay()
+  torch.cuda.synchronize()
+  assert torch.equal(again, first)
+
+
+# ---- torch.compile through the default backend ------------------------------------------------------------
+@pytest.mark.parametrize("quantize_activation", [False, True])
+def test_q_linear_module_inductor(ops, quantize_activation):
+  # test_quantized_matmul.py:128-143 (test_q_linear_module_dynamo) with torch.compile's default backend
+  from xla_amd.quantization import quantize_linear
+  torch.manual_seed(0)
+  with torch.no_grad():
+    lin = torch.nn.Linear(512, 256, bias=False)
+    x = torch.randn(3, 512)
+    q = quantize_linear(lin, n_bits=8, quantize_activation=quantize_activation)
+    out_quant = q(x)
+    qd = q.cuda()
+    before = sum(ops.counters.values())
+    torch._dynamo.reset()
+    out_compiled = torch.compile(qd, backend="inductor", fullgraph=True)(x.cuda())
+    assert sum(ops.counters.values()) > before  # a HIP kernel of this library ran
+    assert torch.allclose(out_compiled.cpu(), out_quant, atol=4e-3)
+
+
+def test_quantized_matmul_int8_inductor(ops):
+  # test_pallas.py:921-948: the operator under torch.compile, table hit and miss, result in x.dtype
+  fn = torch.compile(lambda x, w, s: torch.ops.xla.quantized_matmul_int8(x, w, s, quantize_activation=True),
+                     backend="inductor", fullgraph=True)
+  torch._dynamo.reset()
+  for (m, n, k) in [(256, 4096, 4096), (192, 320, 256)]:
+    x = cases.outlier_activations(m, k, torch.bfloat16, seed=41)
+    _, w, s, _ = cases.per_channel_int8(1, n, k, torch.bfloat16, torch.float32, seed=42)
+    eager = torch.ops.xla.quantized_matmul_int8(x.cuda(), w.cuda(), s.cuda(), quantize_activation=True)
+    out = fn(x.cuda(), w.cuda(), s.cuda())
+    assert out.dtype == torch.bfloat16 and torch.equal(out, eager)

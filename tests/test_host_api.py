@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
   for n in names:
     assert hasattr(lib, n), f"{n} declared in the header but not exported"
   assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-  assert lib.xla_amd_qmm_abi_version() == 2
+  assert lib.xla_amd_qmm_abi_version() == 3
 
 
 def test_header_cites_reference_for_each_entry_point():
@@ -78,7 +78,7 @@ def test_error_codes_without_gpu():
   assert lib.xla_amd_qmm_tiled_bytes(17, 256, 8) == 32 * 256
   assert lib.xla_amd_qmm_tiled_bytes(16, 128, 4) == 16 * 64
   assert lib.xla_amd_qmm_tiled_bytes(16, 64, 8) == 0
-  rc = lib.xla_amd_qmm_weight_only_skinny(None, None, None, None, None, 1, 1, 128, 128, 8, 1, 1, 1, 1, None)
+  rc = lib.xla_amd_qmm_weight_only_skinny(None, None, None, None, None, 1, 1, 128, 128, 8, 1, 1, 1, 1, 1, 1, None)
   assert rc == _lib.EINVAL and b"null" in lib.xla_amd_qmm_last_error()
   rc = lib.xla_amd_qmm_quantize_per_token(None, None, None, None, 1, 1, 0, 0, 0, None)
   assert rc == _lib.EINVAL
@@ -86,6 +86,12 @@ def test_error_codes_without_gpu():
   assert rc == _lib.EINVAL
   with pytest.raises(RuntimeError, match="failed"):
     _lib.check(rc, "w8a8_gemm")
+  assert lib.xla_amd_qmm_w8a8_linear_workspace_bytes(2048, 14336, 4096) >= 2048 * 4096 + 2 * 2048 * 4
+  assert lib.xla_amd_qmm_w8a8_linear_workspace_bytes(3, 8, 5) % 256 == 0
+  rc = lib.xla_amd_qmm_w8a8_linear(None, None, None, None, None, None, 0, 1, 1, 16, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, None)
+  assert rc == _lib.EINVAL and b"null" in lib.xla_amd_qmm_last_error()
+  rc = lib.xla_amd_qmm_untile_weight(None, None, 1, 128, 16, 0, 8, None)
+  assert rc == _lib.EINVAL
 
 
 def test_ops_are_registered_with_reference_schemas(qmm):
@@ -97,15 +103,81 @@ def test_ops_are_registered_with_reference_schemas(qmm):
                        "Tensor? quant_block_size=None, bool quantize_activation=False, int? batch_block_size=None")
 
 
-def test_cpu_tensors_take_the_eager_formulation(qmm):
-  x, w, s, _ = cases.per_channel_int8(4, 16, 32, torch.float32, torch.float32, seed=1)
-  z = torch.randn(16, generator=cases.gen(2)) * 0.01
-  assert torch.equal(torch.ops.xla.quantized_matmul(x, w, s, z), oracle.quantized_matmul(x, w, s, z))
-  xb, wb, sb, zb, _ = cases.blockwise(3, 8, 32, 8, 8, torch.float32, seed=3)
-  assert torch.equal(torch.ops.xla.quantized_matmul(xb, wb, sb, zb, block_size=8),
-                     oracle.quantized_matmul(xb, wb, sb, zb, block_size=8))
-  out = torch.ops.xla.quantized_matmul(x, w, s, quantize_activation=True)
-  assert torch.equal(out, oracle.quantized_matmul(x, w, s, quantize_activation=True, overflow="wrap"))
+def _gold():
+  import json
+  return json.load(open(os.path.join(ROOT, "tests", "golden", "quantized_matmul_golden.json")))
+
+
+def _bf16_from_bits(bits):
+  import numpy as np
+  return torch.tensor(np.asarray(bits, dtype=np.uint16).astype(np.int32)).to(torch.int16).view(torch.bfloat16)
+
+
+def test_cpu_tensors_against_fixtures_and_the_exact_model(qmm):
+  # the CPU key is checked against data that shares no code with it: the hand-worked fixtures, the exact
+  # integer / float64 model, and the reference's fake-quant identity
+  import numpy as np
+  from oracle import bitexact_model as bx
+  op = torch.ops.xla.quantized_matmul
+  g = _gold()["hand_per_channel"]
+  x, w = torch.tensor(g["x"]), torch.tensor(g["w"], dtype=torch.int8)
+  s, z = torch.tensor(g["scale"]), torch.tensor(g["zp"])
+  assert torch.equal(op(x, w, s), torch.tensor(g["expect"]))
+  assert torch.equal(op(x, w, s, z), torch.tensor(g["expect_zp"]))
+  g = _gold()["hand_blockwise"]
+  x, w = torch.tensor(g["x"]), torch.tensor(g["w"], dtype=torch.int8)
+  s, z = torch.tensor(g["scale"]), torch.tensor(g["zp"])
+  assert torch.equal(op(x, w, s, block_size=2), torch.tensor(g["expect"]))
+  assert torch.equal(op(x, w, s, z, block_size=2), torch.tensor(g["expect_zp"]))
+  # W8A8: quantizer and accumulators from the exact model, epilogue as written in the operator's contract
+  x = cases.outlier_activations(32, 512, torch.bfloat16, seed=7)
+  _, w, s, _ = cases.per_channel_int8(1, 48, 512, torch.bfloat16, torch.float32, seed=8)
+  q, xs, _ = bx.quantize_rows(x.double().numpy(), "bf16", "saturate")
+  acc = torch.tensor(bx.int_matmul(q, w.numpy()))
+  expect = (acc.float() * s) * torch.tensor(xs, dtype=torch.float32)[:, None]
+  out = op(x, w, s, quantize_activation=True)
+  assert out.dtype == torch.float32 and torch.equal(out, expect)
+  zp = torch.randn(48, generator=cases.gen(9)) * 0.01
+  xsum = torch.tensor(q.sum(-1), dtype=torch.float32)[:, None]
+  expect_zp = (acc.float() * s - xsum * zp) * torch.tensor(xs, dtype=torch.float32)[:, None]
+  assert torch.equal(op(x, w, s, zp, quantize_activation=True), expect_zp)
+  # blockwise asymmetric: x @ (w * scale - zp) in float64 (test_quantized_matmul.py:210-218)
+  xb, wb, sb, zb, _ = cases.blockwise(6, 24, 64, 16, 4, torch.float32, symmetric=False, seed=2)
+  ref = bx.dense_fake_quant(xb.numpy(), wb.permute(2, 0, 1).reshape(24, 64).numpy(), sb.numpy(), zb.numpy(), 16)
+  assert np.abs(op(xb, wb, sb, zb, block_size=16).double().numpy() - ref).max() < 1e-5
+  # bf16 weight-only: dot rounded to bf16, then scaled and rounded again
+  x, w, s, _ = cases.per_channel_int8(16, 256, 1024, torch.bfloat16, torch.bfloat16, seed=6)
+  two = ((x.double() @ w.double().T).to(torch.bfloat16).float() * s.float()).to(torch.bfloat16)
+  out = op(x, w, s)
+  assert out.dtype == torch.bfloat16 and cases.rel_l2(out, two) < 3e-4
+  # batch dimensions, and agreement with the restatement of the reference's op sequence within tolerance
+  x3 = torch.randn(2, 3, 64, generator=cases.gen(3))
+  assert op(x3, wb, sb, zb, block_size=16).shape == (2, 3, 24)
+  assert cases.within_tolerance(op(x3, wb, sb, zb, block_size=16), oracle.quantized_matmul(x3, wb, sb, zb, block_size=16))
+
+
+def test_cpu_key_follows_the_overflow_policy(qmm, monkeypatch):
+  # one operator, one answer: CPU tensors apply the float -> int8 policy of the GPU kernels
+  g = _gold()["bf16_overflow_band"]
+  x = _bf16_from_bits(g["maxima_bits"]).reshape(-1, 1)
+  ident = torch.ones(1, 1, dtype=torch.int8)
+  one = torch.ones(1)
+  for policy in ("saturate", "wrap"):
+    monkeypatch.setenv("XLA_AMD_QMM_OVERFLOW", policy)
+    q, s = qmm._quantize_tensor(x)
+    assert q.flatten().tolist() == g["q_" + policy]
+    assert torch.equal(s.flatten(), _bf16_from_bits(g["scale_bits"]))
+    # through the operator: out = q * 1 * x_scale
+    out = torch.ops.xla.quantized_matmul(x, ident, one, quantize_activation=True)
+    assert torch.equal(out.flatten(), torch.tensor(g["q_" + policy], dtype=torch.float32) * s.flatten().float())
+  monkeypatch.delenv("XLA_AMD_QMM_OVERFLOW")
+  assert qmm._overflow_policy() == "saturate"
+  q, _ = qmm._quantize_tensor(x)
+  assert q.flatten().tolist() == g["q_saturate"]
+  z, zs = qmm._quantize_tensor(torch.zeros(2, 8, dtype=torch.bfloat16))
+  assert z.abs().sum() == 0 and zs.abs().sum() == 0
+  n, ns = qmm._quantize_tensor(torch.tensor([[1.0, float("nan"), 2.0]]))
+  assert n.abs().sum() == 0 and torch.isnan(ns).all()
 
 
 def test_meta_tensors(qmm):
@@ -153,7 +225,7 @@ def test_module_matches_reference_layout(qmm):
   with pytest.raises(AssertionError):
     mb.load_quantized_weight(torch.zeros(8, 6, dtype=torch.int8), torch.rand(3, 8))
   x = torch.randn(4, 6)
-  assert torch.equal(mb(x), oracle.quantized_matmul(x, mb.weight, mb.weight_scaler, mb.zero_point, block_size=2))
+  assert torch.allclose(mb(x), oracle.quantized_matmul(x, mb.weight, mb.weight_scaler, mb.zero_point, block_size=2), atol=1e-6)
 
 
 def test_rtn_quantizer_and_module_swap(qmm):

@@ -166,6 +166,42 @@ def test_w8a8_integer_model():
   assert p.dtype == torch.bfloat16 and torch.equal(p, expect.to(torch.bfloat16))
 
 
+def test_dedicated_kernel_float_branch():
+  # oracle.quantized_matmul_int8(quantize_activation=False), the float branch of the reference's dedicated kernel
+  # (quantized_matmul_kernel.py:108-121, :246): float32 accumulation, * float32 scale, ONE cast to x.dtype
+  x, w, s, _ = cases.per_channel_int8(16, 256, 1024, torch.bfloat16, torch.bfloat16, seed=6)
+  out = oracle.quantized_matmul_int8(x, w, s)
+  assert out.dtype == torch.bfloat16
+  exact = (x.double() @ w.double().T) * s.float().double()  # the scale enters as float32 (:219-221)
+  one = exact.to(torch.bfloat16)
+  # bf16(f64 dot * scale) within one ulp everywhere (f32 accumulation can flip a tie), equal almost everywhere
+  ulp = torch.ldexp(torch.ones_like(exact), torch.frexp(exact.abs().clamp_min(1e-30))[1].to(torch.int32) - 8)
+  assert ((out.double() - exact).abs() <= ulp).all()
+  assert (out == one).float().mean() > 0.99
+  # one rounding, not two: closer to the exact result than the quantized_matmul sequence (dot -> bf16, * scale -> bf16)
+  two = oracle.quantized_matmul(x, w, s)
+  assert cases.rel_l2(out, exact) < 0.8 * cases.rel_l2(two, exact)
+  # w == 1: row sums times scale; one-hot x: a weight column times scale, exactly
+  ones = torch.ones(7, 1024, dtype=torch.int8)
+  s7 = torch.rand(7, generator=cases.gen(2))
+  rs = oracle.quantized_matmul_int8(x, ones, s7)
+  assert torch.equal(rs, ((x.double().sum(-1, keepdim=True)).float() * s7).to(torch.bfloat16))
+  e = torch.zeros(1, 1024, dtype=torch.bfloat16)
+  e[0, 9] = 1.0
+  assert torch.equal(oracle.quantized_matmul_int8(e, w, s)[0], (w[:, 9].float() * s.float()).to(torch.bfloat16))
+  # float32 activations: nothing is rounded in between, both operators agree
+  xf, wf, sf, _ = cases.per_channel_int8(5, 48, 256, torch.float32, torch.float32, seed=4)
+  assert torch.equal(oracle.quantized_matmul_int8(xf, wf, sf), oracle.quantized_matmul(xf, wf, sf))
+
+
+def test_quantizer_nan_and_zero_rows():
+  x = torch.tensor([[1.0, float("nan"), -2.0, 0.5], [0.0, 0.0, 0.0, 0.0], [1.0, 2.0, -4.0, 0.25]]).bfloat16()
+  q, s = oracle.quantize_tensor(x)
+  assert q[0].abs().sum() == 0 and torch.isnan(s[0]).all()      # NaN row: scale NaN (torch.amax), values 0
+  assert q[1].abs().sum() == 0 and s[1].item() == 0.0           # zero row
+  assert q[2].tolist() == [32, 64, -127, 8]
+
+
 def test_output_dtypes():
   x = torch.randn(3, 8).bfloat16()
   w = torch.randint(-8, 8, (5, 8), dtype=torch.int8)

@@ -26,6 +26,7 @@ SOURCES = [
     ("qmm_quant_act.hip", [], "qmm_quant_act.o"),
     ("qmm_qdq.hip", [], "qmm_qdq.o"),
     ("qmm_w8a8_gemm.hip", [], "qmm_w8a8_gemm.o"),
+    ("qmm_linear.hip", [], "qmm_linear.o"),
 ]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -49,7 +50,7 @@ def _run(cmd):
   return out
 
 
-def build(verbose: bool = False, jobs: int = 7) -> str:
+def build(verbose: bool = False, jobs: int = 8) -> str:
   os.makedirs(OBJ_DIR, exist_ok=True)
   objs = []
 

@@ -19,6 +19,17 @@ int qmm_check_hip(hipError_t e, const char* what) {
   return qmm_fail(XLA_AMD_QMM_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+int qmm_set_max_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done, const char* what) {
+  int dev = 0;
+  int rc = qmm_check_hip(hipGetDevice(&dev), what);
+  if (rc != XLA_AMD_QMM_OK) return rc;
+  const uint64_t bit = dev >= 0 && dev < 64 ? (1ull << dev) : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return XLA_AMD_QMM_OK;
+  rc = qmm_check_hip(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes), what);
+  if (rc == XLA_AMD_QMM_OK && bit) done.fetch_or(bit, std::memory_order_release);
+  return rc;
+}
+
 extern "C" int xla_amd_qmm_abi_version(void) { return XLA_AMD_QMM_ABI_VERSION; }
 
 extern "C" const char* xla_amd_qmm_last_error(void) { return g_err; }

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "xla_amd_qmm.h"
 
 // ---- host side -------------------------------------------------------------
@@ -13,6 +15,12 @@ int qmm_fail(int code, const char* fmt, ...);
 int qmm_check_hip(hipError_t e, const char* what);
 // Error of the launch that was just issued on the calling thread.
 #define QMM_CHECK_LAUNCH(what) qmm_check_hip(hipGetLastError(), what)
+
+// Raises a kernel's dynamic-LDS limit (hipFuncAttributeMaxDynamicSharedMemorySize) once per
+// device: the attribute belongs to the function as loaded on the current device, so `done`
+// (one mask per kernel instantiation, shared by all host threads) holds one bit per device
+// ordinal; ordinals from 64 on set the attribute on every launch.
+int qmm_set_max_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done, const char* what);
 
 static inline bool qmm_valid_dt(int dt) { return dt >= XLA_AMD_DT_F32 && dt <= XLA_AMD_DT_F16; }
 static inline int qmm_dt_size(int dt) { return dt == XLA_AMD_DT_F32 ? 4 : 2; }

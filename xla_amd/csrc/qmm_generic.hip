@@ -9,11 +9,14 @@
 //   o     = round_o( sum_s scale[s,n] * p_s )
 //   zpo   = round_z( sum_s round_x(sum_c x[m,s,c]) * zp[s,n] ),  o = round_o(o - zpo)
 // With S == 1 this is the per-channel formula round_o(round_x(dot) * scale[n]).
+// dot_dt replaces x's dtype in the rounding of p_s (f32: the dot product is not rounded);
+// the result is stored as store_dt (out_dt, or a final cast of it).
 __global__ void __launch_bounds__(256)
 qmm_weight_only_generic_kernel(const void* __restrict__ x, const int8_t* __restrict__ w,
                                const void* __restrict__ scale, const void* __restrict__ zp,
                                void* __restrict__ out, int64_t M, int64_t N, int64_t K, int64_t C,
-                               int w_layout, int x_dt, int scale_dt, int zp_dt, int out_dt) {
+                               int w_layout, int x_dt, int scale_dt, int zp_dt, int dot_dt, int out_dt,
+                               int store_dt) {
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= M * N) return;
   int64_t m = idx / N, n = idx % N;
@@ -29,26 +32,29 @@ qmm_weight_only_generic_kernel(const void* __restrict__ x, const int8_t* __restr
       acc = fmaf(xv, (float)wv, acc);
       xs += xv;
     }
-    float p = qmm_round_dt(acc, x_dt);
+    float p = qmm_round_dt(acc, dot_dt);
     o = fmaf(qmm_load(scale, s * N + n, scale_dt), p, o);
     if (zp) zacc = fmaf(qmm_round_dt(xs, x_dt), qmm_load(zp, s * N + n, zp_dt), zacc);
   }
   o = qmm_round_dt(o, out_dt);
   if (zp) o = qmm_round_dt(o - qmm_round_dt(zacc, zpo_dt), out_dt);
-  qmm_store(out, idx, o, out_dt);
+  qmm_store(out, idx, o, store_dt);
 }
 
 extern "C" int xla_amd_qmm_weight_only_generic(const void* x, const int8_t* w, const void* scale,
                                                const void* zp, void* out, int64_t M, int64_t N,
                                                int64_t K, int64_t C, int w_layout, int x_dt,
-                                               int scale_dt, int zp_dt, int out_dt, void* stream) {
+                                               int scale_dt, int zp_dt, int dot_dt, int out_dt,
+                                               int store_dt, void* stream) {
   if (!x || !w || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_generic: null pointer");
   if (M < 0 || N <= 0 || K <= 0 || C <= 0 || K % C != 0)
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_generic: bad sizes M=%lld N=%lld K=%lld C=%lld",
                     (long long)M, (long long)N, (long long)K, (long long)C);
-  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) ||
-      (zp && !qmm_valid_dt(zp_dt)))
+  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || !qmm_valid_dt(dot_dt) ||
+      !qmm_valid_dt(store_dt) || (zp && !qmm_valid_dt(zp_dt)))
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_generic: bad dtype enum");
+  if (dot_dt != x_dt && (dot_dt != XLA_AMD_DT_F32 || C != K))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_generic: dot dtype must be x's, or f32 for per-channel weights");
   if (w_layout != XLA_AMD_W_NK && w_layout != XLA_AMD_W_SCN)
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_generic: bad weight layout %d", w_layout);
   if (w_layout == XLA_AMD_W_NK && C != K)
@@ -61,7 +67,7 @@ extern "C" int xla_amd_qmm_weight_only_generic(const void* x, const int8_t* w, c
   if (blocks > 0x7fffffffLL) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_generic: too many outputs");
   hipLaunchKernelGGL(qmm_weight_only_generic_kernel, dim3((unsigned)blocks), dim3(256), 0,
                      (hipStream_t)stream, x, w, scale, zp, out, M, N, K, C, w_layout, x_dt,
-                     scale_dt, zp_dt, out_dt);
+                     scale_dt, zp_dt, dot_dt, out_dt, store_dt);
   return QMM_CHECK_LAUNCH("weight_only_generic launch");
 }
 
@@ -198,6 +204,54 @@ extern "C" int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, 
   hipLaunchKernelGGL(qmm_tile_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, w,
                      (i32x4*)tiled, N, K, src_layout, bits, total);
   return QMM_CHECK_LAUNCH("tile_weight launch");
+}
+
+// Inverse of qmm_tile_kernel: one thread reads the 16 bytes of one lane fragment and writes
+// the 16 (bits 8) or 32 (bits 4) weights they hold back into the operator's layout.
+__global__ void __launch_bounds__(256)
+qmm_untile_kernel(const i32x4* __restrict__ tiled, int8_t* __restrict__ w, int64_t N, int64_t K,
+                  int dst_layout, int bits, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int chunks = bits == 8 ? 128 : 64;
+  const int c = (int)(idx % chunks);
+  const int64_t blk = idx / chunks;
+  const int64_t n_blk = K / 128;
+  const int64_t t = blk % n_blk, g = blk / n_blk;
+  const int l = c & 63, h = c >> 6;
+  const int64_t n = 16 * g + (l & 15);
+  if (n >= N) return;
+  const int64_t k0 = 128 * t + 32 * (l >> 4) + 16 * h;
+  const i32x4 v = tiled[idx];
+  auto put = [&](int64_t k, int val) {
+    if (dst_layout == XLA_AMD_W_NK) w[n * K + k] = (int8_t)val;
+    else w[k * N + n] = (int8_t)val;
+  };
+  if (bits == 8) {
+    for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < 4; ++j) put(k0 + 4 * i + j, (int)(int8_t)((uint32_t)v[i] >> (8 * j)));
+  } else {
+    const int P[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+    for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < 8; ++j) put(k0 + 8 * i + P[j], (int)(((uint32_t)v[i] >> (4 * j)) & 15u) - 8);
+  }
+}
+
+extern "C" int xla_amd_qmm_untile_weight(const void* tiled, int8_t* w, int64_t S, int64_t C, int64_t N,
+                                         int dst_layout, int bits, void* stream) {
+  if (!w || !tiled) return qmm_fail(XLA_AMD_QMM_EINVAL, "untile_weight: null pointer");
+  if (S <= 0 || C <= 0 || N <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "untile_weight: bad sizes");
+  if (bits != 4 && bits != 8) return qmm_fail(XLA_AMD_QMM_EINVAL, "untile_weight: bits must be 4 or 8");
+  if (dst_layout != XLA_AMD_W_NK && dst_layout != XLA_AMD_W_SCN)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "untile_weight: bad layout %d", dst_layout);
+  const int64_t K = S * C;
+  if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "untile_weight: K=%lld not a multiple of 128", (long long)K);
+  const int64_t total = ((N + 15) / 16) * (K / 128) * (bits == 8 ? 128 : 64);
+  const int64_t blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffLL) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "untile_weight: weight too large");
+  hipLaunchKernelGGL(qmm_untile_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const i32x4*)tiled, w, N, K, dst_layout, bits, total);
+  return QMM_CHECK_LAUNCH("untile_weight launch");
 }
 
 extern "C" int xla_amd_qmm_pack_weight(const int8_t* w, void* packed, int64_t S, int64_t C, int64_t N,

@@ -1,0 +1,72 @@
+// Operator-level entry points of the W8A8 path: per-token activation quantization
+// followed by the int8 GEMM, in one call.  The quantized activations (x_q, their
+// scales and row sums) are intermediate device memory, taken from a caller-provided
+// workspace.
+#include "qmm_common.h"
+
+namespace {
+
+constexpr size_t kAlign = 256;
+constexpr size_t round_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+// Layout of the intermediate memory for an [M, K] activation:
+//   x_q     int8  [M, K]   at 0
+//   x_scale 4-byte slots [M] (f32, or bf16/f16 in the low half) after it
+//   x_sum   int32 [M]      after that
+struct Carve {
+  size_t xq, scale, sum, total;
+};
+Carve carve(int64_t M, int64_t K) {
+  Carve c;
+  c.xq = 0;
+  c.scale = round_up((size_t)M * (size_t)K);
+  c.sum = c.scale + round_up((size_t)M * 4);
+  c.total = c.sum + round_up((size_t)M * 4);
+  return c;
+}
+
+int run_linear(const void* x, const int8_t* w, const void* w_scale, const void* zp, void* out,
+               unsigned char* mem, const Carve& c, int64_t M, int64_t N, int64_t K, int x_dt,
+               int w_scale_dt, int zp_dt, int x_scale_dt, int cvt_dt, int mid_dt, int out_dt,
+               int overflow_policy, int block_m, int block_n, void* stream) {
+  int8_t* xq = (int8_t*)(mem + c.xq);
+  void* xs = mem + c.scale;
+  int32_t* xsum = zp ? (int32_t*)(mem + c.sum) : nullptr;
+  int rc = xla_amd_qmm_quantize_per_token(x, xq, xs, xsum, M, K, x_dt, x_scale_dt, overflow_policy, stream);
+  if (rc != XLA_AMD_QMM_OK) return rc;
+  return xla_amd_qmm_w8a8_gemm(xq, w, xs, w_scale, zp, xsum, out, nullptr, M, N, K, x_scale_dt, w_scale_dt,
+                               zp_dt, cvt_dt, mid_dt, zp_dt, out_dt, block_m, block_n, stream);
+}
+
+int check_common(const char* who, const void* x, const int8_t* w, const void* w_scale, void* out, int64_t M,
+                 int64_t N, int64_t K) {
+  if (!x || !w || !w_scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "%s: null pointer", who);
+  if (M < 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "%s: bad sizes M=%lld N=%lld K=%lld", who,
+                                                 (long long)M, (long long)N, (long long)K);
+  if (M > (1 << 30) || N > (1 << 30) || K > (1 << 30)) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "%s: dimension too large", who);
+  return XLA_AMD_QMM_OK;
+}
+
+}  // namespace
+
+extern "C" size_t xla_amd_qmm_w8a8_linear_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  (void)N;
+  if (M < 0 || K <= 0) return 0;
+  return carve(M, K).total;
+}
+
+extern "C" int xla_amd_qmm_w8a8_linear(const void* x, const int8_t* w, const void* w_scale, const void* zp,
+                                       void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                                       int64_t K, int x_dt, int w_scale_dt, int zp_dt, int x_scale_dt,
+                                       int cvt_dt, int mid_dt, int out_dt, int overflow_policy, int block_m,
+                                       int block_n, void* stream) {
+  int rc = check_common("w8a8_linear", x, w, w_scale, out, M, N, K);
+  if (rc != XLA_AMD_QMM_OK) return rc;
+  if (M == 0) return XLA_AMD_QMM_OK;
+  const Carve c = carve(M, K);
+  if (!workspace || workspace_bytes < c.total)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_linear: workspace of %zu bytes, need %zu", workspace ? workspace_bytes : (size_t)0, c.total);
+  if ((uintptr_t)workspace & (kAlign - 1)) return qmm_fail(XLA_AMD_QMM_EINVAL, "w8a8_linear: workspace must be 256-byte aligned");
+  return run_linear(x, w, w_scale, zp, out, (unsigned char*)workspace, c, M, N, K, x_dt, w_scale_dt, zp_dt,
+                    x_scale_dt, cvt_dt, mid_dt, out_dt, overflow_policy, block_m, block_n, stream);
+}

@@ -3,6 +3,9 @@
 // registers between the abs-max pass and the quantize pass (x is read exactly
 // once); longer rows are read a second time, which hits L2.
 //
+// A row that holds a NaN: scale = NaN (torch.amax propagates it), every x_q of the row 0
+// (the reference's cast of NaN to int8 is undefined).  An all-zero row: scale = 0, x_q = 0.
+//
 // The arithmetic is the reference's, op by op, in x's dtype:
 //   max = amax(|x|); scale = RN_x(max / 127); r = RN_x(x / scale); q = int8(rint(r))
 // RN_x(a / b) is obtained as RN_x(RN_f32(a / b)): a and b carry at most 11
@@ -14,9 +17,11 @@ namespace {
 
 constexpr int kThreads = 256;
 
+// max that keeps a NaN (fmaxf would drop it): a row that holds a NaN gets a NaN scale, as torch.amax gives
+__device__ __forceinline__ float nan_max(float a, float b) { return (a > b || a != a) ? a : b; }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  for (int o = 32; o > 0; o >>= 1) v = nan_max(v, __shfl_xor(v, o, 64));
   return v;
 }
 __device__ __forceinline__ int wave_sum(int v) {
@@ -82,8 +87,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
         load_vec(k, held[s]);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) {
-          float av = fabsf(held[s][i]);
-          mx = (av > mx || av != av) ? av : mx;
+          mx = nan_max(fabsf(held[s][i]), mx);
         }
       }
     }
@@ -93,8 +97,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
       load_vec(k, f);
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
-        float av = fabsf(f[i]);
-        mx = (av > mx || av != av) ? av : mx;  // propagate NaN like torch.amax
+        mx = nan_max(fabsf(f[i]), mx);
       }
     }
   }
@@ -103,7 +106,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
   __syncthreads();
   mx = smax[0];
 #pragma unroll
-  for (int i = 1; i < kThreads / 64; ++i) mx = fmaxf(mx, smax[i]);
+  for (int i = 1; i < kThreads / 64; ++i) mx = nan_max(mx, smax[i]);
   const float scale = qmm_round_dt(mx / 127.0f, XT);
 
   // pass 2: quantize

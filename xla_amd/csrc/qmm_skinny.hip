@@ -50,6 +50,8 @@ struct SkinnyArgs {
   void* out;
   int M, N, K, C;  // M = rows of this pass (<= 16*MT)
   int scale_dt, zp_dt, out_dt;
+  int dot_dt;    // dtype the dot product is rounded to before it is scaled (per-channel only)
+  int store_dt;  // dtype of the stored tensor (out_dt, or a final cast of it)
 };
 
 int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
@@ -188,6 +190,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int K = a.K, N = a.N, M = a.M, C = a.C;
   const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
   const int x_dt = XT;
+  // (blockwise launches always round the block dot products to x's dtype: a compile-time constant there)
+  const int dot_dt = RED == kRedRaw ? a.dot_dt : XT;
 
   // ---- weights: global -> registers, already in MFMA operand order ------------------
   // The tiled weight holds, for every group of 16 channels and every sub-step of
@@ -357,7 +361,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
         const float xsv = NEEDXS ? xs[mt][v] : 0.f;
-        const float p = qmm_round_dt(true_dot(acc[mt][v] + accb[mt][v], xsv), x_dt);
+        const float p = qmm_round_dt(true_dot(acc[mt][v] + accb[mt][v], xsv), dot_dt);
         sacc[mt][v] = fmaf(sc, p, sacc[mt][v]);
         if constexpr (HASZP) zacc[mt][v] = fmaf(qmm_round_dt(xsv, x_dt), zv, zacc[mt][v]);
       });
@@ -604,12 +608,14 @@ qmm_skinny_kernel(SkinnyArgs a) {
         o2 = qmm_round_dt(o2 - qmm_round_dt(zacc[mt][2], zpo_dt), a.out_dt);
         o3 = qmm_round_dt(o3 - qmm_round_dt(zacc[mt][3], zpo_dt), a.out_dt);
       }
+      // (a store dtype narrower than out_dt is the caller's final cast: one more rounding, done by the conversion)
+      const int st = a.store_dt;
       const size_t idx = (size_t)m * N + n;
       if ((N & 3) == 0) {  // 4 consecutive channels: one aligned 8- or 16-byte store
-        if (a.out_dt == XLA_AMD_DT_F32) {
+        if (st == XLA_AMD_DT_F32) {
           *(f32x4*)((float*)a.out + idx) = f32x4{o0, o1, o2, o3};
         } else {
-          const bool bf = a.out_dt == XLA_AMD_DT_BF16;
+          const bool bf = st == XLA_AMD_DT_BF16;
           const uint32_t h0 = bf ? qmm_f32_to_bf16(o0) : qmm_f32_to_f16(o0);
           const uint32_t h1 = bf ? qmm_f32_to_bf16(o1) : qmm_f32_to_f16(o1);
           const uint32_t h2 = bf ? qmm_f32_to_bf16(o2) : qmm_f32_to_f16(o2);
@@ -617,10 +623,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
           *(i32x2*)((uint16_t*)a.out + idx) = i32x2{(int)(h0 | (h1 << 16)), (int)(h2 | (h3 << 16))};
         }
       } else {
-        qmm_store(a.out, idx, o0, a.out_dt);
-        if (n + 1 < N) qmm_store(a.out, idx + 1, o1, a.out_dt);
-        if (n + 2 < N) qmm_store(a.out, idx + 2, o2, a.out_dt);
-        if (n + 3 < N) qmm_store(a.out, idx + 3, o3, a.out_dt);
+        qmm_store(a.out, idx, o0, st);
+        if (n + 1 < N) qmm_store(a.out, idx + 1, o1, st);
+        if (n + 2 < N) qmm_store(a.out, idx + 2, o2, st);
+        if (n + 3 < N) qmm_store(a.out, idx + 3, o3, st);
       }
     }
   });
@@ -633,13 +639,9 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: tile does not fit in LDS");
   } else {
     auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, NW, WSEG>;
-    static thread_local bool attr_set = false;
-    if (!attr_set) {
-      int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 Cfg::lds_bytes(Cfg::CHG)), "weight_only_skinny hipFuncSetAttribute");
-      if (rc != XLA_AMD_QMM_OK) return rc;
-      attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_set{0};
+    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(Cfg::CHG), lds_set, "weight_only_skinny hipFuncSetAttribute");
+    if (rc != XLA_AMD_QMM_OK) return rc;
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
     const int steps = (a.K + Cfg::KS - 1) / Cfg::KS;
     hipLaunchKernelGGL(kern, dim3(blocks), dim3(NW * 64), Cfg::lds_bytes(steps), stream, a);
@@ -708,16 +710,20 @@ int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_
 extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const void* scale,
                                               const void* zp, void* out, int64_t M, int64_t N,
                                               int64_t K, int64_t C, int bits, int x_dt, int scale_dt,
-                                              int zp_dt, int out_dt, void* stream) {
+                                              int zp_dt, int dot_dt, int out_dt, int store_dt,
+                                              void* stream) {
   if (!x || !w_tiled || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: null pointer");
   if (M < 0 || N <= 0 || K <= 0 || C <= 0 || K % C != 0)
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: bad sizes M=%lld N=%lld K=%lld C=%lld",
                     (long long)M, (long long)N, (long long)K, (long long)C);
   if (bits != 4 && bits != 8) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: bits must be 4 or 8");
-  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || (zp && !qmm_valid_dt(zp_dt)))
+  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || !qmm_valid_dt(dot_dt) ||
+      !qmm_valid_dt(store_dt) || (zp && !qmm_valid_dt(zp_dt)))
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: bad dtype enum");
   if (out_dt != qmm_promote(x_dt, scale_dt))
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: out dtype must be promote(x, scale)");
+  if (dot_dt != x_dt && (dot_dt != XLA_AMD_DT_F32 || C != K))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_skinny: dot dtype must be x's, or f32 for per-channel weights");
   if (K % 128 != 0 || C % 128 != 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: K=%lld and C=%lld must be multiples of 128",
                     (long long)K, (long long)C);
@@ -732,7 +738,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
   if (((uintptr_t)out & 15) && (N & 3) == 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: out must be 16-byte aligned");
   if (M == 0) return XLA_AMD_QMM_OK;
-  const int xsz = qmm_dt_size(x_dt), osz = qmm_dt_size(out_dt);
+  const int xsz = qmm_dt_size(x_dt), osz = qmm_dt_size(store_dt);
   const int pass = x_dt == XLA_AMD_DT_F32 ? 16 : 32;  // rows of x per pass over the weight
   for (int64_t m0 = 0; m0 < M; m0 += pass) {
     SkinnyArgs a;
@@ -744,6 +750,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
     a.M = (int)((M - m0) < pass ? (M - m0) : pass);
     a.N = (int)N; a.K = (int)K; a.C = (int)C;
     a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.out_dt = out_dt;
+    a.dot_dt = dot_dt; a.store_dt = store_dt;
     int rc;
     if (x_dt == XLA_AMD_DT_BF16) rc = qmm_skinny_launch_bf16(a, bits, zp != nullptr, (hipStream_t)stream);
     else if (x_dt == XLA_AMD_DT_F16) rc = qmm_skinny_launch_f16(a, bits, zp != nullptr, (hipStream_t)stream);

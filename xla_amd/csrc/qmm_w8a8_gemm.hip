@@ -436,13 +436,9 @@ int launch_tile_epi(GemmArgs g, hipStream_t stream) {
   constexpr size_t lds = KG * NS * (size_t)(BM + BN) * kBK;
   static_assert(lds <= 160 * 1024 && KG * WM * WN * 64 <= 1024, "workgroup must fit a CU");
   auto kern = qmm_w8a8_gemm_kernel<BM, BN, WM, WN, EPI, NS, KG>;
-  static thread_local bool attr_set = false;
-  if (!attr_set) {
-    int rc = qmm_check_hip(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds),
-                           "w8a8_gemm hipFuncSetAttribute");
-    if (rc != XLA_AMD_QMM_OK) return rc;
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_set{0};
+  const int rc = qmm_set_max_lds((const void*)kern, (int)lds, lds_set, "w8a8_gemm hipFuncSetAttribute");
+  if (rc != XLA_AMD_QMM_OK) return rc;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(KG * WM * WN * 64), lds, stream, g);
   return QMM_CHECK_LAUNCH("w8a8_gemm launch");
 }

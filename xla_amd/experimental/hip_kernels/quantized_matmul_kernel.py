@@ -1,13 +1,66 @@
-"""Tuned workgroup tiles of the gfx950 W8A8 GEMM, by problem shape.
+"""The dedicated int8 kernel and its tuned workgroup tiles, by problem shape.
 
-Plays the role of TUNED_BLOCK_SIZES / get_tuned_block_sizes in
-torch_xla/experimental/pallas_kernels/quantized_matmul_kernel.py:326-555: a
-table from (device generation, batch, out features, in features, activation
-dtype, quantize_activation) to the block sizes the kernel is launched with.
-Here a "block" is the output tile of one workgroup (batch_block x out_block)
-and the K extent of one LDS pipeline stage (in_block).
+Counterpart of torch_xla/experimental/pallas_kernels/quantized_matmul_kernel.py:
+`quantized_matmul_int8` (:171-310) launches the gfx950 kernels with the
+arithmetic of the Pallas `matmul_kernel` (:88-124), and TUNED_BLOCK_SIZES /
+get_tuned_block_sizes (:326-555) map (device generation, batch, out features,
+in features, activation dtype, quantize_activation) to the block sizes the
+kernel is launched with.  Here a "block" is the output tile of one workgroup
+(batch_block x out_block) and the K extent of one LDS pipeline stage (in_block).
 """
 import torch
+
+from xla_amd import _lib
+
+
+def quantized_matmul_int8(
+    x: torch.Tensor,  # [bs, n_input_features]
+    w: torch.Tensor,  # [n_output_features, n_input_features] int8
+    scalar: torch.Tensor,  # [n_output_features]
+    zero_point=None,
+    quant_block_size=None,
+    quantize_activation: bool = False,
+    *,
+    batch_block_size=None,
+    out_block_size=None,
+    in_block_size=None,
+):
+  """int8-weight matmul with the arithmetic of the reference's dedicated kernel; result in x.dtype.
+
+  quantize_activation: row abs-max, activation scale and quotient in x.dtype
+  (:10-18, :199-200), int32 accumulation, then `acc * w_scale * x_scale` in
+  float32 and one cast (:117-121).  Otherwise the float branch (:108-112,
+  :246): float32 accumulation over all of K, `acc * w_scale` in float32, one
+  cast.  The weight scale is always taken as float32 (:219-221).
+
+  All three block sizes must be given, as in the reference (:194).  A
+  (batch, out) pair the GEMM has no workgroup tile for, and `in_block_size`
+  (the K extent of a pipeline stage is fixed at 128), act as hints only: the
+  library then chooses the tile by shape; block sizes never change a value.
+  """
+  from xla_amd.experimental import xla_quantized_matmul as _qmm
+  assert zero_point is None, "Not implemented: zero_point is not supported."
+  assert quant_block_size is None, "Not implemented: quant_block_size is not supported."
+  assert batch_block_size is not None and out_block_size is not None and in_block_size is not None
+  assert x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], (
+      f"x.shape[1] ({x.shape[1]}) must be equal to w.shape[1] ({w.shape[1]})")
+  assert w.shape[0] == scalar.shape[0], (
+      f"w.shape[0] ({w.shape[0]}) must be equal to scalar.shape[0] ({scalar.shape[0]})")
+  x2 = x.contiguous()
+  w = w.contiguous()
+  scalar32 = scalar.to(torch.float32).contiguous()
+  if quantize_activation:
+    if (batch_block_size, out_block_size) not in _SUPPORTED_TILES:
+      batch_block_size = out_block_size = 0
+    return _qmm.w8a8_linear_gpu(x2, w, scalar32, None, x_scale_dtype=torch.float32, cvt_dtype=torch.float32,
+                                mid_dtype=torch.float32, out_dtype=x.dtype, block_m=batch_block_size,
+                                block_n=out_block_size)
+  return _qmm._weight_only_gpu(x2, w, scalar32, None, -1, False, torch.float32, dot_dtype=torch.float32,
+                               store_dtype=x.dtype)
+
+
+# workgroup tiles (batch_block, out_block) the W8A8 GEMM is built for
+_SUPPORTED_TILES = ((32, 32), (64, 32), (64, 64), (128, 128), (128, 256), (256, 256))
 
 _ARCH = "gfx950"
 

@@ -9,6 +9,8 @@ kernels through libxla_amd_qmm.so; values follow torch's own decomposition
 The argument checks are the reference's `_check_scale_zp` (:52-70) plus its
 "all scales > 0" assertion (:86-87).
 """
+import weakref
+
 import torch
 from torch.library import impl
 # defines the quantized_decomposed operators and their CPU / Meta implementations
@@ -19,14 +21,28 @@ from xla_amd import _lib
 _QDT = {torch.int8: _lib.QDT_I8, torch.uint8: _lib.QDT_U8, torch.int16: _lib.QDT_I16, torch.int32: _lib.QDT_I32}
 
 
+# Parameter tensors whose values have been checked: (id(scale), id(zero_point), dtype) ->
+# (versions and storage pointers at the time).  The value checks need the numbers on the host,
+# which synchronises the device for GPU parameters; they run once per pair of parameter tensors,
+# so that repeated calls with the same parameters launch without a synchronisation and can be
+# captured into a HIP graph.
+_validated = {}
+
+
+def _param_state(t):
+  try:
+    v = t._version
+  except RuntimeError:
+    v = -1
+  return (v, t.data_ptr(), t.numel())
+
+
 def _check_scale_zp(input, scale, zero_point, axis, dtype):
   # 1. scale, zp are 1-D; 2. their length matches the (de)quant dim or is 1;
   # 3. dtype is an integer type; 4. zero points lie within dtype's range
   assert len(scale.shape) == 1 and len(zero_point.shape) == 1
   assert 'int' in str(dtype)
   assert dtype in _QDT, f"xla_amd: quantized dtype {dtype} is not supported on the GPU path"
-  info = torch.iinfo(dtype)
-  assert torch.equal(zero_point.cpu(), torch.clamp(zero_point.cpu(), info.min, info.max))
   if axis == -1:
     assert scale.numel() == 1 and zero_point.numel() == 1
   else:
@@ -34,8 +50,23 @@ def _check_scale_zp(input, scale, zero_point, axis, dtype):
     qdq_dim_size = input.shape[axis]
     assert qdq_dim_size == scale.numel() or scale.numel() == 1
     assert qdq_dim_size == zero_point.numel() or zero_point.numel() == 1
+  key = (id(scale), id(zero_point), dtype)
+  state = (_param_state(scale), _param_state(zero_point))
+  if _validated.get(key) == state:
+    return
+  if (scale.is_cuda or zero_point.is_cuda) and torch.cuda.is_current_stream_capturing():
+    raise RuntimeError("xla_amd: quantization parameters are checked on the host the first time they are "
+                       "seen; call the operator once with these parameter tensors before capturing a graph")
+  info = torch.iinfo(dtype)
+  zp_host = zero_point.cpu()
+  assert torch.equal(zp_host, torch.clamp(zp_host, info.min, info.max))
   # all scales must be greater than 0 (StableHLO qdq constraint the reference enforces)
-  assert bool((scale > 0).all())
+  assert bool((scale.cpu() > 0).all())
+  if len(_validated) > 1024:
+    _validated.clear()
+  _validated[key] = state
+  for t in (scale, zero_point):
+    weakref.finalize(t, _validated.pop, key, None)
 
 
 def _check_scalar(scale, zero_point, dtype):
@@ -45,6 +76,18 @@ def _check_scalar(scale, zero_point, dtype):
   info = torch.iinfo(dtype)
   assert info.min <= zero_point <= info.max
   assert scale > 0
+
+
+def _per_channel_params(input, axis, scale, zero_point):
+  """scale and zero_point with one entry per channel of `axis` (either may come with a single entry),
+  or both with a single entry."""
+  n = max(scale.numel(), 1 if zero_point is None else zero_point.numel())
+  if n > 1:
+    assert n == input.shape[axis]
+    scale = scale.expand(n)
+    if zero_point is not None:
+      zero_point = zero_point.expand(n)
+  return scale, zero_point
 
 
 def _geometry(input, axis, n_params):
@@ -128,6 +171,7 @@ def rocm_quantize_per_channel(input: torch.Tensor, scales: torch.Tensor, zero_po
   _float_input(input)
   assert axis < input.dim(), f"Expecting axis to be < {input.dim()}"
   _check_scale_zp(input, scales, zero_points, axis, dtype)
+  scales, zero_points = _per_channel_params(input, axis, scales, zero_points)
   inv = 1.0 / scales.to(torch.float32) if scales.dtype != torch.float64 else (1.0 / scales).to(torch.float32)
   return _quantize(input, inv, zero_points, quant_min, quant_max, dtype, axis)
 
@@ -146,4 +190,5 @@ def rocm_dequantize_per_channel(input: torch.Tensor, scales: torch.Tensor, zero_
   assert axis < input.dim(), f"Expecting axis to be < {input.dim()}"
   zp_check = zero_points if zero_points is not None else torch.zeros_like(scales, dtype=torch.int64)
   _check_scale_zp(input, scales, zp_check, axis, dtype)
+  scales, zero_points = _per_channel_params(input, axis, scales, zero_points)
   return _dequantize(input, scales, zero_points, dtype, out_dtype, axis, 1)

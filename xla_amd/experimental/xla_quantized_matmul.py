@@ -3,15 +3,15 @@
 Drop-in for torch_xla/experimental/xla_quantized_matmul.py: same operator
 schema (:7-9), same shape/dtype checks and messages (:12-53), same module
 (:186-243).  Tensors on a ROCm GPU run hand-written gfx950 kernels through
-libxla_amd_qmm.so; there is no fallback for them.  CPU tensors take the
-reference's own eager formulation (:139-183), which the reference documents
-as its debugging path; meta tensors only get shapes and dtypes.
+libxla_amd_qmm.so; there is no fallback for them.  CPU tensors take an eager
+formulation with the rounding points of the reference's (:139-183), which the
+reference documents as its debugging path; meta tensors only get shapes and
+dtypes.
 """
 import os
 import weakref
 
 import torch
-import torch.nn.functional as F
 from torch.library import impl
 
 from xla_amd import _lib
@@ -92,16 +92,50 @@ def _result_dtype(x, scaler, quantize_activation):
 
 
 # ---- one-time re-layouts of weights ----------------------------------------------
-# key (id(w), kind) -> (version, data_ptr, bits, copy); dropped when w dies.
+# The streaming kernel reads a tiled copy of the weight (blocks of 16 channels x
+# 128 columns in MFMA operand order).  It is made once per weight tensor, either
+# explicitly (`prepare_weight`, `XlaQuantizedLinear.prepare`) or on the first call
+# that needs it, and kept in `_pack_cache` while the tensor object is alive.
+#
+# key (id(w), kind) -> (version, data_ptr, bits, copy)
 _pack_cache = {}
+
+
+def _version_of(w: torch.Tensor) -> int:
+  try:
+    return w._version
+  except RuntimeError:  # inference tensors do not track a version counter
+    return -1
+
+
+def invalidate_weight_cache(w: torch.Tensor = None):
+  """Drops the cached re-layouts of `w` (of every weight when `w` is None).
+
+  The cache notices in-place operations on the weight through torch's version
+  counter.  Writes that bypass the counter are invisible to it and need this
+  call: `w.data.copy_(...)` / `w.data[...] = ...`, anything written into an
+  inference-mode tensor, and writes from outside torch to the same memory.
+  """
+  if w is None:
+    _pack_cache.clear()
+    return
+  for kind in ("tiled", "packed"):
+    _pack_cache.pop((id(w), kind), None)
 
 
 def _relayout(w: torch.Tensor, bits: int, layout: int, kind: str) -> torch.Tensor:
   key = (id(w), kind)
   hit = _pack_cache.get(key)
-  if hit is not None and hit[0] == w._version and hit[1] == w.data_ptr() and hit[2] == bits:
+  if hit is not None and hit[0] == _version_of(w) and hit[1] == w.data_ptr() and hit[2] == bits:
     counters["pack_hit"] += 1
     return hit[3]
+  if torch.cuda.is_current_stream_capturing():
+    # The copy would only be recorded, not made: the buffer would stay empty until the first
+    # replay and every replay would repeat the re-layout.
+    raise RuntimeError(
+        "xla_amd: the weight of a quantized_matmul call has no device-side copy yet and the current "
+        "stream is being captured into a HIP graph; call xla_amd.experimental.xla_quantized_matmul."
+        "prepare_weight(w, ...) or XlaQuantizedLinear.prepare() (or run the call once) before the capture")
   if layout == _lib.W_NK:
     n, k = w.shape
     s, c = 1, k
@@ -119,7 +153,7 @@ def _relayout(w: torch.Tensor, bits: int, layout: int, kind: str) -> torch.Tenso
   counters["pack"] += 1
   if hit is None:
     weakref.finalize(w, _pack_cache.pop, key, None)
-  _pack_cache[key] = (w._version, w.data_ptr(), bits, out)
+  _pack_cache[key] = (_version_of(w), w.data_ptr(), bits, out)
   return out
 
 
@@ -133,46 +167,81 @@ def _tiled_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
 
   The copy is made once per weight tensor and reused while the tensor is alive
   and unmodified (same object, same storage pointer, same version counter); it
-  costs as much device memory again as the weight itself.
+  costs as much device memory again as the weight itself (half for int4).
   """
   return _relayout(w, bits, layout, "tiled")
 
 
-def _weight_only_gpu(x2, w, scaler, zero_point, block_size, int4_weight, out_dtype):
+def _weight_geometry(w, block_size):
+  """(n, k, c, layout) of an operator weight."""
+  if block_size == -1:
+    n, k = w.shape
+    return n, k, k, _lib.W_NK
+  s, c, n = w.shape
+  return n, s * c, c, _lib.W_SCN
+
+
+def prepare_weight(w: torch.Tensor, block_size: int = -1, int4_weight: bool = False, x_dtype=torch.bfloat16):
+  """Makes the device-side copy of `w` that `quantized_matmul(x, w, ...)` will read, now.
+
+  Returns True when the weight-only call for this weight runs the streaming
+  kernel (which reads a tiled copy), False when it reads `w` itself and there is
+  nothing to prepare.  Call it before capturing a HIP graph: the first call for a
+  weight otherwise makes the copy lazily, which a capture must not record.
+  """
+  if not w.is_cuda:
+    return False
+  n, k, c, layout = _weight_geometry(w, block_size)
+  bits = 4 if int4_weight else 8
+  if _lib.load().xla_amd_qmm_dispatch(1, n, k, c, bits, _lib.dt(x_dtype), 0) != _lib.KERNEL_SKINNY_MFMA:
+    return False
+  _tiled_weight(w.contiguous() if not w.is_contiguous() else w, bits, layout)
+  return True
+
+
+def _weight_only_launch(x2, w, w_tiled, n, k, c, layout, bits, scaler, zero_point, out_dtype, dot_dtype, store_dtype):
+  """One weight-only launch; `w` (operator layout) or `w_tiled` may be None, not both."""
   lib = _lib.load()
-  m, k = x2.shape
-  blockwise = block_size != -1
-  n = w.shape[-1] if blockwise else w.shape[0]
-  c = block_size if blockwise else k
+  m = x2.shape[0]
+  blockwise = c != k
   if blockwise and (scaler.dtype != x2.dtype or (zero_point is not None and zero_point.dtype != x2.dtype)):
     # torch.einsum / torch.matmul of the reference raise on mixed dtypes here
     raise RuntimeError(
         f"expected scalar type {x2.dtype} for blockwise scaler/zero_point, got {scaler.dtype}"
         f"{'' if zero_point is None else '/' + str(zero_point.dtype)}")
-  out = torch.empty((m, n), dtype=out_dtype, device=x2.device)
+  dot_dtype = dot_dtype or x2.dtype
+  store_dtype = store_dtype or out_dtype
+  out = torch.empty((m, n), dtype=store_dtype, device=x2.device)
   if m == 0:
     return out
-  bits = 4 if int4_weight else 8
   kern = lib.xla_amd_qmm_dispatch(m, n, k, c, bits, _lib.dt(x2.dtype), 0)
-  layout = _lib.W_SCN if blockwise else _lib.W_NK
   stream = _lib.stream_of(x2)
   zp_dt = _lib.dt(zero_point.dtype) if zero_point is not None else _lib.dt(x2.dtype)
+  dts = (_lib.dt(x2.dtype), _lib.dt(scaler.dtype), zp_dt, _lib.dt(dot_dtype), _lib.dt(out_dtype),
+         _lib.dt(store_dtype))
   if kern == _lib.KERNEL_SKINNY_MFMA:
-    wk = _tiled_weight(w, bits, layout)
+    wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
     counters["skinny_mfma"] += 1
     _lib.check(
         lib.xla_amd_qmm_weight_only_skinny(x2.data_ptr(), wk.data_ptr(), scaler.data_ptr(),
                                            _lib.ptr(zero_point), out.data_ptr(), m, n, k, c, bits,
-                                           _lib.dt(x2.dtype), _lib.dt(scaler.dtype), zp_dt,
-                                           _lib.dt(out_dtype), stream), "weight_only_skinny")
+                                           *dts, stream), "weight_only_skinny")
   else:
+    if w is None:
+      raise RuntimeError("xla_amd: this shape runs the generic kernel, which reads the operator's weight layout")
     counters["generic"] += 1
     _lib.check(
         lib.xla_amd_qmm_weight_only_generic(x2.data_ptr(), w.data_ptr(), scaler.data_ptr(),
                                             _lib.ptr(zero_point), out.data_ptr(), m, n, k, c, layout,
-                                            _lib.dt(x2.dtype), _lib.dt(scaler.dtype), zp_dt,
-                                            _lib.dt(out_dtype), stream), "weight_only_generic")
+                                            *dts, stream), "weight_only_generic")
   return out
+
+
+def _weight_only_gpu(x2, w, scaler, zero_point, block_size, int4_weight, out_dtype, dot_dtype=None,
+                     store_dtype=None):
+  n, k, c, layout = _weight_geometry(w, block_size)
+  return _weight_only_launch(x2, w, None, n, k, c, layout, 4 if int4_weight else 8, scaler, zero_point,
+                             out_dtype, dot_dtype, store_dtype)
 
 
 def quantize_per_token_gpu(x2: torch.Tensor, scale_dtype=None, want_sum=False, overflow=None):
@@ -214,6 +283,55 @@ def w8a8_gemm_gpu(x_q, w, x_scale, w_scale, zero_point, x_sum, *, cvt_dtype, mid
   return out, acc
 
 
+def quantized_matmul_gpu(x, w, scaler, zero_point=None, block_size=-1, int4_weight=False,
+                         quantize_activation=False, store_dtype=None):
+  """`quantized_matmul` on ROCm tensors; `store_dtype` fuses a final `.to(store_dtype)` of the result."""
+  block_size = -1 if block_size is None else block_size
+  int4_weight = bool(int4_weight)
+  quantize_activation = bool(quantize_activation)
+  _check_args(x, w, scaler, zero_point, block_size, quantize_activation)
+  if not (x.is_floating_point() and scaler.is_floating_point()):
+    raise RuntimeError(f"xla_amd quantized_matmul: x and scaler must be floating point, got {x.dtype}, {scaler.dtype}")
+  out_dtype = _result_dtype(x, scaler, quantize_activation)
+  x2 = x.reshape(-1, x.shape[-1]).contiguous()
+  w = w.contiguous()
+  scaler = scaler.contiguous()
+  if zero_point is not None:
+    zero_point = zero_point.contiguous()
+  if quantize_activation:
+    out = w8a8_linear_gpu(x2, w, scaler, zero_point, x_scale_dtype=x2.dtype, cvt_dtype=scaler.dtype,
+                          mid_dtype=scaler.dtype, out_dtype=out_dtype)
+    if store_dtype is not None and store_dtype != out_dtype:
+      out = out.to(store_dtype)
+  else:
+    out = _weight_only_gpu(x2, w, scaler, zero_point, block_size, int4_weight, out_dtype, store_dtype=store_dtype)
+  return out.reshape(*x.shape[:-1], out.shape[-1])
+
+
+def w8a8_linear_gpu(x2, w, w_scale, zero_point, *, x_scale_dtype, cvt_dtype, mid_dtype, out_dtype, overflow=None,
+                    block_m=0, block_n=0):
+  """Per-token quantization + int8 GEMM in one library call; the quantized activations live in a workspace
+  that is only needed during the call (the caching allocator hands the same block to the next call)."""
+  lib = _lib.load()
+  m, k = x2.shape
+  n = w.shape[0]
+  out = torch.empty((m, n), dtype=out_dtype, device=x2.device)
+  if m == 0:
+    return out
+  nbytes = lib.xla_amd_qmm_w8a8_linear_workspace_bytes(m, n, k)
+  workspace = torch.empty(nbytes, dtype=torch.uint8, device=x2.device)
+  kern = lib.xla_amd_qmm_dispatch(m, n, k, k, 8, _lib.DT_F32, 1)
+  counters["w8a8_mfma" if kern == _lib.KERNEL_W8A8_MFMA else "w8a8_generic"] += 1
+  zp_dt = _lib.dt(zero_point.dtype) if zero_point is not None else _lib.DT_F32
+  _lib.check(
+      lib.xla_amd_qmm_w8a8_linear(x2.data_ptr(), w.data_ptr(), w_scale.data_ptr(), _lib.ptr(zero_point),
+                                  out.data_ptr(), workspace.data_ptr(), nbytes, m, n, k, _lib.dt(x2.dtype),
+                                  _lib.dt(w_scale.dtype), zp_dt, _lib.dt(x_scale_dtype), _lib.dt(cvt_dtype),
+                                  _lib.dt(mid_dtype), _lib.dt(out_dtype), _OVERFLOW[overflow or _overflow_policy()],
+                                  block_m, block_n, _lib.stream_of(x2)), "w8a8_linear")
+  return out
+
+
 @impl(XLA_LIB, "quantized_matmul", "CUDA")
 def quantized_matmul_rocm(x: torch.Tensor,
                           w: torch.Tensor,
@@ -234,34 +352,63 @@ def quantized_matmul_rocm(x: torch.Tensor,
          per byte once per weight tensor.
       quantize_activation: per-token dynamic int8 quantization of x (W8A8).
   """
-  block_size = -1 if block_size is None else block_size
-  int4_weight = bool(int4_weight)
-  quantize_activation = bool(quantize_activation)
-  _check_args(x, w, scaler, zero_point, block_size, quantize_activation)
-  if not (x.is_floating_point() and scaler.is_floating_point()):
-    raise RuntimeError(f"xla_amd quantized_matmul: x and scaler must be floating point, got {x.dtype}, {scaler.dtype}")
-  out_dtype = _result_dtype(x, scaler, quantize_activation)
-  x2 = x.reshape(-1, x.shape[-1]).contiguous()
-  w = w.contiguous()
-  scaler = scaler.contiguous()
-  if zero_point is not None:
-    zero_point = zero_point.contiguous()
-  if quantize_activation:
-    x_q, x_scale, x_sum = quantize_per_token_gpu(x2, want_sum=zero_point is not None)
-    out, _ = w8a8_gemm_gpu(x_q, w, x_scale, scaler, zero_point, x_sum, cvt_dtype=scaler.dtype,
-                           mid_dtype=scaler.dtype, out_dtype=out_dtype)
+  return quantized_matmul_gpu(x, w, scaler, zero_point, block_size, int4_weight, quantize_activation)
+
+
+# ---- CPU tensors --------------------------------------------------------------------
+# The reference documents calls with CPU tensors as its debugging path
+# (docs/source/perf/quantized_ops.md:48-49) and its CI compares the device against it.
+# The formulation below is this package's own; it rounds to the tensor dtype at exactly
+# the points where the reference's op sequence (:139-183) materialises a tensor, and it
+# applies the same explicit float -> int8 overflow policy as the GPU kernels, so that a
+# CPU tensor and a GPU tensor give the same answer.
+
+
+def _quantize_tensor(x: torch.Tensor, n_bits: int = 8, dim: int = -1, overflow: str = None):
+  """Per-token symmetric quantizer (:56-73): every step is one torch op in x's dtype.
+
+  Returns (int8 values, scale in x's dtype, kept dim).  A quotient that rounds to
+  +-2^(n_bits-1) (the scale is itself rounded) follows the overflow policy; an
+  all-zero row gives zeros with scale 0, a row with a NaN gives zeros with scale NaN.
+  """
+  qmax = (1 << (n_bits - 1)) - 1
+  scale = x.abs().amax(dim=dim, keepdim=True) / qmax
+  r = torch.nan_to_num((x / scale).round().float(), nan=0.0, posinf=0.0, neginf=0.0)
+  policy = overflow or _overflow_policy()
+  if policy == "saturate":
+    q = r.clamp(-qmax - 1, qmax).to(torch.int8)
   else:
-    out = _weight_only_gpu(x2, w, scaler, zero_point, block_size, int4_weight, out_dtype)
-  return out.reshape(*x.shape[:-1], out.shape[-1])
+    q = r.to(torch.int32).to(torch.int8)  # modulo 256, what torch's own cast does
+  return q, scale.to(x.dtype)
 
 
-def _quantize_tensor(x: torch.Tensor, n_bits: int = 8, dim: int = -1):
-  """Eager form of the activation quantizer (:56-73), used for CPU tensors."""
-  max_val = torch.amax(torch.abs(x), dim=dim, keepdim=True)
-  int_max = 2**(n_bits - 1) - 1
-  scale = max_val / int_max
-  x_int = torch.round(x / scale).to(torch.int8)
-  return x_int, scale.to(x.dtype)
+def _cpu_per_channel(x2, w, scaler, zero_point, quantize_activation):
+  if quantize_activation:
+    x_q, x_scale = _quantize_tensor(x2)
+    acc = torch.mm(x_q.to(torch.int32), w.to(torch.int32).t())  # exact
+    out = acc * scaler  # integer tensor times float tensor: converted to scaler's dtype first
+    if zero_point is not None:
+      row_sum = x_q.to(torch.int32).sum(dim=-1, keepdim=True)
+      out.sub_(row_sum * zero_point)
+    return out * x_scale
+  out = torch.mm(x2, w.to(x2.dtype).t()) * scaler
+  if zero_point is not None:
+    out.sub_(x2.sum(dim=-1, keepdim=True) * zero_point)
+  return out
+
+
+def _cpu_blockwise(x2, w, scaler, zero_point, block_size):
+  m = x2.shape[0]
+  s, c, n = w.shape
+  xb = x2.reshape(m, s, c)
+  # per block: [s, m, c] @ [s, c, n] -> [s, m, n], rounded to x's dtype
+  p = torch.bmm(xb.transpose(0, 1), w.to(x2.dtype))
+  # sum over blocks of scaler[s, n] * p[s, m, n] as one contraction per channel (a single rounding)
+  out = torch.bmm(p.permute(2, 1, 0), scaler.t().unsqueeze(-1)).squeeze(-1).t()
+  if zero_point is not None:
+    out = out.contiguous()
+    out.sub_(torch.mm(xb.sum(dim=-1), zero_point))
+  return out
 
 
 @impl(XLA_LIB, "quantized_matmul", "CPU")
@@ -272,31 +419,16 @@ def quantized_matmul(x: torch.Tensor,
                      block_size: int = -1,
                      int4_weight: bool = False,
                      quantize_activation: bool = False):
-  """CPU tensors only: the reference's eager debugging path (:139-183)."""
+  """CPU tensors (the reference's debugging path, :139-183); `int4_weight` only concerns storage."""
   block_size = -1 if block_size is None else block_size
+  quantize_activation = bool(quantize_activation)
   _check_args(x, w, scaler, zero_point, block_size, quantize_activation)
+  x2 = x.reshape(-1, x.shape[-1])
   if block_size == -1:
-    w = w.to(x.dtype)
-    if quantize_activation:
-      x, x_scale = _quantize_tensor(x)
-      x = x.to(torch.int32)
-      w = w.to(torch.int32)
-    out = F.linear(x, w)
-    out = out * scaler
+    out = _cpu_per_channel(x2, w, scaler, zero_point, quantize_activation)
   else:
-    x = x.reshape(*x.shape[:-1], x.shape[-1] // block_size, block_size)
-    w = w.to(x.dtype)
-    out = torch.einsum('scn,...sc->...sn', w, x)
-    out = torch.einsum('sn,...sn->...n', scaler, out)
-  if zero_point is not None:
-    if block_size == -1:
-      zp_out = torch.einsum("...c,z->...z", x, zero_point)
-    else:
-      zp_out = torch.matmul(x.sum(dim=-1), zero_point)
-    out -= zp_out
-  if quantize_activation:
-    out = out * x_scale
-  return out
+    out = _cpu_blockwise(x2, w, scaler, zero_point, block_size)
+  return out.reshape(*x.shape[:-1], out.shape[-1])
 
 
 @impl(XLA_LIB, "quantized_matmul", "Meta")
@@ -309,12 +441,48 @@ def quantized_matmul_meta(x, w, scaler, zero_point=None, block_size=-1, int4_wei
                      device=x.device)
 
 
+# ---- weight-only matmul on a tiled weight alone ----------------------------------------
+# Not part of the reference's interface: the operator a module calls once it keeps only the
+# tiled form of its weight on the device (XlaQuantizedLinear.prepare(release_weight=True)).
+XLA_AMD_LIB = torch.library.Library("xla_amd", "DEF")
+XLA_AMD_LIB.define(
+    "weight_only_tiled(Tensor x, Tensor w_tiled, Tensor scale, Tensor? zero_point, int out_features, "
+    "int block_size, bool int4_weight) -> Tensor")
+
+
+@impl(XLA_AMD_LIB, "weight_only_tiled", "CUDA")
+def weight_only_tiled_rocm(x, w_tiled, scaler, zero_point, out_features, block_size, int4_weight):
+  if not (x.is_floating_point() and scaler.is_floating_point()):
+    raise RuntimeError(f"xla_amd weight_only_tiled: x and scaler must be floating point, got {x.dtype}, {scaler.dtype}")
+  k = x.shape[-1]
+  c = k if block_size == -1 else block_size
+  bits = 4 if int4_weight else 8
+  need = _lib.load().xla_amd_qmm_tiled_bytes(out_features, k, bits)
+  assert need > 0 and w_tiled.numel() * w_tiled.element_size() == need, (
+      f"tiled weight of {w_tiled.numel() * w_tiled.element_size()} bytes does not belong to a "
+      f"[{out_features}, {k}] weight of {bits} bits")
+  x2 = x.reshape(-1, k).contiguous()
+  out = _weight_only_launch(x2, None, w_tiled, out_features, k, c, _lib.W_NK if c == k else _lib.W_SCN, bits,
+                            scaler.contiguous(), None if zero_point is None else zero_point.contiguous(),
+                            _result_dtype(x, scaler, False), None, None)
+  return out.reshape(*x.shape[:-1], out_features)
+
+
+@impl(XLA_AMD_LIB, "weight_only_tiled", "Meta")
+def weight_only_tiled_meta(x, w_tiled, scaler, zero_point, out_features, block_size, int4_weight):
+  return torch.empty(*x.shape[:-1], out_features, dtype=_result_dtype(x, scaler, False), device=x.device)
+
+
 class XlaQuantizedLinear(torch.nn.Module):
   """Linear layer over a quantized weight (xla_quantized_matmul.py:186-243).
 
   State-dict keys and buffer shapes are the reference's: `weight` int8
   [out, in], `weight_scaler` [out], and `zero_point` [out] unless symmetric;
   `load_quantized_weight` replaces them (blockwise weights are 3-D).
+
+  On a ROCm GPU, `prepare()` makes the tiled copy of the weight that the
+  streaming kernel reads ahead of the first forward, and can drop the
+  reference-layout buffer from device memory; `state_dict()` still returns it.
   """
 
   def __init__(self,
@@ -337,6 +505,11 @@ class XlaQuantizedLinear(torch.nn.Module):
       self.register_buffer('zero_point', torch.zeros(output_dim))
     else:
       self.zero_point = None
+    # tiled copy owned by the module (set by prepare(); moves with .to()/.cuda(), never saved)
+    self.register_buffer('_weight_tiled', None, persistent=False)
+    self._released_shape = None  # shape of `weight` while only the tiled form is kept
+    self._tiled_from = None      # (version, storage pointer) of `weight` when the tiled copy was made
+    self._register_state_dict_hook(XlaQuantizedLinear._restore_weight_in_state_dict)
 
   def load_quantized_weight(self, weight, weight_scaler, zero_point=None):
     '''
@@ -353,8 +526,80 @@ class XlaQuantizedLinear(torch.nn.Module):
     self.weight = weight
     self.weight_scaler = weight_scaler
     self.zero_point = zero_point
+    self._weight_tiled = None
+    self._released_shape = None
+
+  # -- device-side weight layout ----------------------------------------------------------
+  def prepare(self, release_weight: bool = False) -> bool:
+    """Makes the tiled copy of the weight now instead of on the first forward.
+
+    Needed before a HIP-graph capture (the lazy copy must not be recorded), and
+    after writes to `weight` that torch's version counter cannot see
+    (`weight.data.copy_`).  Returns False when this layer does not use a tiled
+    copy (CPU tensors, activation quantization, shapes of the generic kernel).
+    With `release_weight=True` the reference-layout `weight` buffer is freed on
+    the device and only the tiled form is kept (half the weight memory);
+    `state_dict()` rebuilds `weight` from it, `load_state_dict()` brings the
+    buffer back (call `prepare` again afterwards).
+    """
+    if self._released_shape is not None:
+      return True
+    w = self.weight
+    if not w.is_cuda or self.quantize_activation:
+      return False
+    n, k, c, layout = _weight_geometry(w, self.block_size)
+    bits = 4 if self.int4_weight else 8
+    if _lib.load().xla_amd_qmm_dispatch(1, n, k, c, bits, _lib.DT_BF16, 0) != _lib.KERNEL_SKINNY_MFMA:
+      return False
+    invalidate_weight_cache(w)
+    self._weight_tiled = _tiled_weight(w.contiguous(), bits, layout)
+    self._tiled_from = (_version_of(w), w.data_ptr())
+    if release_weight:
+      invalidate_weight_cache(w)  # the module's own reference keeps the copy alive
+      self._released_shape = tuple(w.shape)
+      self.weight = torch.empty(0, dtype=torch.int8, device=w.device)
+    return True
+
+  def _rebuilt_weight(self):
+    shape = self._released_shape
+    if len(shape) == 2:
+      (n, k), s, c, layout = shape, 1, shape[1], _lib.W_NK
+    else:
+      (s, c, n), layout = shape, _lib.W_SCN
+    w = torch.empty(shape, dtype=torch.int8, device=self._weight_tiled.device)
+    _lib.check(
+        _lib.load().xla_amd_qmm_untile_weight(self._weight_tiled.data_ptr(), w.data_ptr(), s, c, n, layout,
+                                              4 if self.int4_weight else 8, _lib.stream_of(w)), "untile_weight")
+    return w
+
+  @staticmethod
+  def _restore_weight_in_state_dict(module, state_dict, prefix, local_metadata):
+    if module._released_shape is not None:
+      state_dict[prefix + "weight"] = module._rebuilt_weight()
+    return state_dict
+
+  def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+    if self._released_shape is not None:
+      self.weight = torch.empty(self._released_shape, dtype=torch.int8, device=self.weight.device)
+      self._weight_tiled = None
+      self._released_shape = None
+    else:
+      self._weight_tiled = None
+    return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+  def _tiled_is_current(self):
+    if self._weight_tiled is None:
+      return False
+    if self._released_shape is not None:
+      return True
+    # `weight` is still there: the copy stands while torch has seen no write to it (an in-place
+    # operation or a new tensor sends the call back to the operator, which re-tiles)
+    return self._tiled_from == (_version_of(self.weight), self.weight.data_ptr())
 
   def forward(self, x):
+    if x.is_cuda and self._tiled_is_current():
+      return torch.ops.xla_amd.weight_only_tiled(x, self._weight_tiled, self.weight_scaler, self.zero_point,
+                                                 self.output_dim, self.block_size, self.int4_weight)
     return torch.ops.xla.quantized_matmul(
         x,
         self.weight,
