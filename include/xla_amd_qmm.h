@@ -239,6 +239,41 @@ int xla_amd_qmm_w8a8_linear(const void* x, const int8_t* w, const void* w_scale,
                             void* stream);
 
 /*
+ * xla_amd_qmm_w8a8_linear without a workspace argument and without any
+ * allocation.  It has no counterpart in the reference; it is for callers that
+ * cannot allocate device memory around the call: code under HIP-graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  The quantized
+ * activations live in a fixed array inside the library's device image (16 MiB
+ * + 64 KiB, held by every GPU the library is loaded on until the process
+ * ends): at most 8192 rows and M * K <= 16 Mi elements
+ * (xla_amd_qmm_w8a8_linear_noalloc_limits), else XLA_AMD_QMM_EUNSUPPORTED.
+ * Apart from the one-time set-up of a device (xla_amd_qmm_init, or the first
+ * call on that device), the call performs no hipMalloc / hipFree and calls no
+ * allocating library routine; outputs are identical to xla_amd_qmm_w8a8_linear.  Every
+ * call on a GPU shares that GPU's array and nothing in it needs clearing
+ * between calls (each call overwrites what it reads); calls that overlap in
+ * time on one GPU (different streams or threads) race on it and must be
+ * serialised by the caller.
+ */
+int xla_amd_qmm_w8a8_linear_noalloc(const void* x, const int8_t* w, const void* w_scale, const void* zp,
+                                    void* out, int64_t M, int64_t N, int64_t K, int x_dt, int w_scale_dt,
+                                    int zp_dt, int x_scale_dt, int cvt_dt, int mid_dt, int out_dt,
+                                    int overflow_policy, int block_m, int block_n, void* stream);
+
+/*
+ * Per-device set-up of the library for the current device: resolves the address
+ * of this GPU's copy of the fixed scratch array (the HIP runtime backs the array
+ * with device memory when it is first looked up).  Optional:
+ * xla_amd_qmm_w8a8_linear_noalloc does the same on its first call on a device.
+ * Call it outside HIP-graph capture.  Safe to call repeatedly and from several
+ * threads.
+ */
+int xla_amd_qmm_init(void);
+
+/* Limits of xla_amd_qmm_w8a8_linear_noalloc: rows of x, and elements M * K of x.  Host pointers, nullable. */
+void xla_amd_qmm_w8a8_linear_noalloc_limits(int64_t* max_rows, int64_t* max_elements);
+
+/*
  * Shape-based choice between the kernels (the role of the tuned-table lookup
  * with fallback in torch_xla/experimental/custom_kernel.py:1088-1106).
  * Pure host function; returns an XLA_AMD_KERNEL_* id.

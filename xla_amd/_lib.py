@@ -38,6 +38,9 @@ SIGNATURES = {
     "xla_amd_qmm_w8a8_gemm": (_c_int, [_c_vp] * 8 + [_c_i64] * 3 + [_c_int] * 9 + [_c_vp]),
     "xla_amd_qmm_w8a8_linear_workspace_bytes": (ctypes.c_size_t, [_c_i64] * 3),
     "xla_amd_qmm_w8a8_linear": (_c_int, [_c_vp] * 6 + [ctypes.c_size_t] + [_c_i64] * 3 + [_c_int] * 10 + [_c_vp]),
+    "xla_amd_qmm_init": (_c_int, []),
+    "xla_amd_qmm_w8a8_linear_noalloc": (_c_int, [_c_vp] * 5 + [_c_i64] * 3 + [_c_int] * 10 + [_c_vp]),
+    "xla_amd_qmm_w8a8_linear_noalloc_limits": (None, [ctypes.POINTER(_c_i64)] * 2),
     "xla_amd_qmm_dispatch": (_c_int, [_c_i64] * 4 + [_c_int] * 3),
     "xla_amd_qmm_w8a8_tile": (_c_int, [_c_i64] * 3 + [ctypes.POINTER(ctypes.c_int32)]),
     "xla_amd_qmm_quantize_affine": (_c_int, [_c_vp] * 4 + [_c_i64] * 3 + [_c_int] * 2 + [ctypes.c_int32] * 2 + [_c_vp]),
