@@ -56,6 +56,14 @@ __device__ __forceinline__ void qmm_lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Workgroup barrier with no fence at all: waits for this wave's own LDS operations, then
+// s_barrier.  For code that keeps global -> LDS copies in flight across the barrier and does
+// its own vmcnt waits (a workgroup-scope fence makes the compiler wait for every such copy,
+// since they are LDS writes); the memory clobber keeps LDS accesses on their side of it.
+__device__ __forceinline__ void qmm_bare_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 __device__ __forceinline__ float qmm_bf16_to_f32(uint16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }

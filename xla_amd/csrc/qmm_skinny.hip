@@ -154,7 +154,6 @@ struct SkinnyCfg {
   static constexpr int BLK = BITS == 8 ? 2048 : 1024;        // bytes of one (16 channels x 128 columns) weight block
   static constexpr int X_TILE = XROWS * XROW;                // the x columns of one step, all rows
   static constexpr int CH = kLdsLimit / X_TILE;              // steps whose x columns are resident in LDS together
-  static constexpr int XPW = X_TILE / 1024 / NW;             // 1 KB pieces of an x tile copied by each wave
   // Steps of weight loads in flight per wave (register ring).  One step is
   // 8 KB per wave, 7 MB over the chip: enough to cover the memory latency; with
   // two or more the measured time goes *up* (the extra requests only queue).
@@ -166,17 +165,25 @@ struct SkinnyCfg {
     const int x = (steps < CHG ? steps : CHG) * X_TILE;
     return x > kRedBytes ? x : kRedBytes;
   }
-  static_assert((X_TILE / 1024) % NW == 0, "x tile must split evenly over the waves");
   static_assert(WSEG == 512 || (WSEG == 256 && BITS == 8), "weight segment");
 };
 
-template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, int NW = kWaves, int WSEG = kWSeg>
-__global__ void __launch_bounds__(NW * 64)
+// Extra waves per workgroup that do nothing but copy x into LDS (see the kernel).  Two waves
+// then share a SIMD and each may use half of its registers: the one configuration that needs
+// more (two x tiles with per-block scale accumulators) runs without them, and its computing
+// waves copy x themselves.
+template <int MT, int RED> constexpr int skinny_copier_waves() { return (MT == 2 && RED != 1 /*kRedRaw*/) ? 0 : 4; }
+
+// UNI: scale, zero point, dot product, result and stored tensor all have x's dtype (the common
+// case, and the only one for blockwise weights): the dtypes are compile-time constants then, and
+// the code that runs once per wave (epilogue, scale conversion) has no dtype branches.
+template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, bool UNI, int NW = kWaves, int WSEG = kWSeg>
+__global__ void __launch_bounds__((NW + skinny_copier_waves<MT, RED>()) * 64)
 qmm_skinny_kernel(SkinnyArgs a) {
   using Cfg = SkinnyCfg<XT, BITS, MT, KW, NW, WSEG>;
   constexpr int NLD = Cfg::NLD;
   constexpr int RW = Cfg::RW, XB = Cfg::XB, KS = Cfg::KS, SUB = Cfg::SUB, XROW = Cfg::XROW;
-  constexpr int X_TILE = Cfg::X_TILE, XPW = Cfg::XPW, P = Cfg::P, BLK = Cfg::BLK;
+  constexpr int X_TILE = Cfg::X_TILE, P = Cfg::P, BLK = Cfg::BLK;
   constexpr bool kMfma = XT != XLA_AMD_DT_F32;
   constexpr bool NEEDXS = HASZP || (BITS == 4 && kMfma);  // x sums: zero point, int4 affine map
   constexpr int XQ = kMfma ? 4 : 8;                       // 16-byte x chunks per lane per sub-step
@@ -190,8 +197,9 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int K = a.K, N = a.N, M = a.M, C = a.C;
   const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
   const int x_dt = XT;
-  // (blockwise launches always round the block dot products to x's dtype: a compile-time constant there)
-  const int dot_dt = RED == kRedRaw ? a.dot_dt : XT;
+  const int scale_dt = UNI ? XT : a.scale_dt, zp_dt = UNI ? XT : a.zp_dt, out_dt = UNI ? XT : a.out_dt;
+  const int dot_dt = UNI ? XT : a.dot_dt, store_dt = UNI ? XT : a.store_dt;
+  static_assert(UNI || RED == kRedRaw, "blockwise launches have a single dtype");
 
   // ---- weights: global -> registers, already in MFMA operand order ------------------
   // The tiled weight holds, for every group of 16 channels and every sub-step of
@@ -204,29 +212,11 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const uint8_t* const w_base = a.w + (size_t)my_group * n_blk * BLK + lane * 16;
   const char* const x_base = (const char*)a.x;
   // x: copied global -> LDS without passing registers (global_load_lds_dwordx4:
-  // lane l of an instruction lands at base + 16 l).  Piece j of this wave is
-  // 1 KB of a step's tile: part of one row, or whole consecutive rows when a row
-  // is shorter.  The XOR swizzle of the tile is applied on the source side: LDS
+  // lane l of an instruction lands at base + 16 l), 1 KB of one row per
+  // instruction.  The XOR swizzle of the tile is applied on the source side: LDS
   // slot c' of a row receives global chunk c' ^ (row % 16).
-  constexpr int kPiecesPerRow = XROW >= 1024 ? XROW / 1024 : 1;
-  constexpr int kRowsPerPiece = XROW >= 1024 ? 1 : 1024 / XROW;
-  constexpr int kLanesPerRow = 64 / kRowsPerPiece;
-  uint32_t x_off[XPW];  // per lane: byte offset of its source chunk from the step's first column of row 0
-  int x_col[XPW];       // per lane: byte column of that chunk within the step
-  int x_lds[XPW];       // uniform: LDS offset of the piece within a tile
-  bool x_used[XPW];     // uniform: the piece holds at least one row below M (rows from M on are never
-                        // stored, so their x is not copied: a decode step of one row copies 1/16 of the tile)
-  qmm_static_for<XPW>([&](auto jc) {
-    constexpr int j = jc;
-    const int q = wave * XPW + j;
-    const int row0 = (q / kPiecesPerRow) * kRowsPerPiece, piece = q % kPiecesPerRow;
-    const int row = row0 + lane / kLanesPerRow;
-    const int m = min(row, M - 1);
-    x_col[j] = ((piece * 64 + lane % kLanesPerRow) ^ (row & 15)) * 16;
-    x_off[j] = (uint32_t)m * (uint32_t)(K * XB) + x_col[j];
-    x_lds[j] = row0 * XROW + piece * 1024;
-    x_used[j] = row0 < M;
-  });
+  constexpr int kPiecesPerRow = XROW / 1024;
+  static_assert(XROW % 1024 == 0, "a step of one x row is a whole number of 1 KB pieces");
 
   const int steps_total = (K + KS - 1) / KS;
   const int my_steps = steps_total > kw ? (steps_total - kw + KW - 1) / KW : 0;
@@ -250,30 +240,96 @@ qmm_skinny_kernel(SkinnyArgs a) {
   auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {
     qmm_static_for<SUB>([&](auto tc) { load_sub(pc, s, tc); });
   };
-  // The x columns of global steps c0 .. c0+nst-1 into the LDS tiles 0 .. nst-1.
+  // The x columns of global steps c0+t0 .. c0+t1-1 into the LDS tiles t0 .. t1-1.  The copying
+  // waves (the extra ones, or all waves when there are none) share the rows below M of every
+  // tile, a row per instruction (rows from
+  // M on are never stored, so their x is not copied: a decode step of one row copies
+  // 1/16 of a tile).  The loops are uniform and free of per-piece conditions: this code
+  // runs once per wave, straight after launch, and every branch in it costs an
+  // instruction fetch that nothing hides.
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
-  auto x_chunk_load = [&](int c0, int nst) __attribute__((always_inline)) {
-    for (int t = 0; t < nst; ++t) {
-      const int gs = c0 + t;
-      const char* const xp = x_base + (size_t)gs * XROW;
-      char* const tile = smem + t * X_TILE;
-      if ((gs + 1) * KS <= K) {
-        qmm_static_for<XPW>([&](auto jc) {
-          constexpr int j = jc;
-          if (x_used[j]) __builtin_amdgcn_global_load_lds((const void*)(xp + x_off[j]), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
-        });
-      } else {
-        // last, partial step: chunks past K re-read the last valid 16 bytes of the row
-        const int x_left = K * XB - gs * XROW;
-        qmm_static_for<XPW>([&](auto jc) {
-          constexpr int j = jc;
-          // x_left >= 256 here, so 0 <= back <= x_col[j] <= x_off[j]
-          const int back = max(x_col[j] + 16 - x_left, 0);
-          if (x_used[j]) __builtin_amdgcn_global_load_lds((const void*)(xp + ((int64_t)x_off[j] - back)), (lds_ptr_t)(tile + x_lds[j]), 16, 0, 0);
-        });
+  const int x_rows = min(M, Cfg::XROWS);
+  constexpr int kCopiers = skinny_copier_waves<MT, RED>();
+  constexpr int kCopyWaves = kCopiers > 0 ? kCopiers : NW;
+  const int copy_wave = kCopiers > 0 ? wave - NW : wave;
+  auto x_chunk_load = [&](int c0, int t0, int t1) __attribute__((always_inline)) {
+    for (int row = copy_wave; row < x_rows; row += kCopyWaves) {
+      const char* xrow = x_base + (size_t)row * ((size_t)K * XB) + (size_t)c0 * XROW;  // row `row`, first column of the chunk
+      char* lrow = smem + row * XROW;
+      const int sw = row & 15;
+      for (int t = t0; t < t1; ++t) {
+        const char* xp = xrow + (size_t)t * XROW;
+        char* dst = lrow + t * X_TILE;
+        if ((c0 + t + 1) * KS <= K) {
+          qmm_static_for<kPiecesPerRow>([&](auto pc) {
+            constexpr int piece = pc;
+            const uint32_t col = (uint32_t)(((piece * 64 + lane) ^ sw) * 16);
+            __builtin_amdgcn_global_load_lds((const void*)(xp + col), (lds_ptr_t)(dst + piece * 1024), 16, 0, 0);
+          });
+        } else {
+          // last, partial step: chunks past K re-read the last valid 16 bytes of the row
+          const int x_left = K * XB - (c0 + t) * XROW;  // >= 256
+          qmm_static_for<kPiecesPerRow>([&](auto pc) {
+            constexpr int piece = pc;
+            const int col = ((piece * 64 + lane) ^ sw) * 16;
+            const int back = max(col + 16 - x_left, 0);  // 0 <= back <= col
+            __builtin_amdgcn_global_load_lds((const void*)(xp + (col - back)), (lds_ptr_t)(dst + piece * 1024), 16, 0, 0);
+          });
+        }
       }
     }
   };
+  // Copying all of x into every compute unit (the same 128 KB for each of them, out of a few L2
+  // slices) takes longer than the first weights take to arrive from memory, so only the x
+  // columns of the first kFirstTiles steps are waited for before step 0; the rest land while
+  // those steps run, and the workgroup meets once more before step kFirstTiles (a multiple
+  // of KW: every wave has the same number of steps before that).
+  //
+  // The computing waves cannot do that themselves: with global -> LDS copies in flight when they
+  // enter the main loop, the compiler can no longer count their loads in flight and turns every
+  // wait of the loop into a wait for all of them.  So kCopiers extra waves do all the copying
+  // and nothing else: they wait for their copies, meet the workgroup at each of its meeting
+  // points, and leave.  The computing waves only request weights.
+  constexpr int CHG = Cfg::CHG;
+  constexpr int kFirstTiles = 4;  // (a multiple of every KW)
+  const int nst0 = min(CHG, steps_total);
+  const bool second_meeting = kCopiers > 0 && nst0 > kFirstTiles;  // uniform over the workgroup
+  if constexpr (kCopiers > 0) {
+    // (marked unlikely so that this block is laid out behind the computing waves' code: they
+    // then run straight on from the kernel's entry to their first loads; a taken branch over
+    // this block would cost them an instruction fetch from memory, the weights of the
+    // previous launch having pushed the code out of L2)
+    if (__builtin_expect(wave >= NW, 0)) {
+      for (int c0 = 0; c0 < steps_total; c0 += CHG) {
+        if (c0 > 0) qmm_bare_barrier();      // every wave has finished reading the old columns
+        const int nst = min(CHG, steps_total - c0);
+        if (c0 == 0 && second_meeting) {
+          x_chunk_load(0, 0, kFirstTiles);
+          __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+          qmm_bare_barrier();
+          x_chunk_load(0, kFirstTiles, nst);
+        } else {
+          x_chunk_load(c0, 0, nst);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        qmm_bare_barrier();
+      }
+      if constexpr (KW > 1) { qmm_bare_barrier(); qmm_bare_barrier(); }  // the two of the k-split reduction
+      return;
+    }
+  }
+
+  // The first step's weights (the longest latency of the kernel: a cold HBM access) go out
+  // before anything else is computed.
+  qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (kCopiers == 0) {
+    // Loads complete in order, so waiting for the copies also waits for those weights, which
+    // step 0 needs anyway.
+    x_chunk_load(0, 0, nst0);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
   // ---- accumulators ----------------------------------------------------------------
   // (register arrays are only ever indexed by compile-time constants: every
   // loop over them is a qmm_static_for)
@@ -300,14 +356,16 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // Per-channel: the only scales a lane ever needs are fetched now, so that
   // their latency is hidden behind the main loop instead of trailing it.
   uint32_t pre_sc[4] = {0u, 0u, 0u, 0u}, pre_zp[4] = {0u, 0u, 0u, 0u};  // raw bits: converted where they are used
-  if constexpr (RED == kRedRaw) {
-    qmm_static_for<4>([&](auto vc) {
-      constexpr int v = vc;
-      const int n = min(n_wave + 4 * g + v, N - 1);
-      pre_sc[v] = qmm_load_raw(a.scale, n, a.scale_dt);
-      if constexpr (HASZP) pre_zp[v] = qmm_load_raw(a.zp, n, a.zp_dt);
-    });
-  }
+  auto fetch_channel_scales = [&]() __attribute__((always_inline)) {
+    if constexpr (RED == kRedRaw) {
+      qmm_static_for<4>([&](auto vc) {
+        constexpr int v = vc;
+        const int n = min(n_wave + 4 * g + v, N - 1);
+        pre_sc[v] = qmm_load_raw(a.scale, n, scale_dt);
+        if constexpr (HASZP) pre_zp[v] = qmm_load_raw(a.zp, n, zp_dt);
+      });
+    }
+  };
   // Blockwise: scale / zero point of 4 consecutive channels are one 16-byte
   // load (8 of them used for 2-byte types), fetched one step ahead: bw_sc[t]
   // holds those of the block that sub-step t of the current step lies in.
@@ -352,8 +410,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
       const int n = min(n_wave + 4 * g + v, N - 1);
       float sc, zv = 0.f;
       if constexpr (RED == kRedRaw) {
-        sc = qmm_from_raw(pre_sc[v], a.scale_dt);
-        if constexpr (HASZP) zv = qmm_from_raw(pre_zp[v], a.zp_dt);
+        sc = qmm_from_raw(pre_sc[v], scale_dt);
+        if constexpr (HASZP) zv = qmm_from_raw(pre_zp[v], zp_dt);
       } else {
         sc = bw_value(bw_sc[t], bw_sc_sel[t], XT, vc);
         if constexpr (HASZP) zv = bw_value(bw_zp[t], bw_zp_sel[t], XT, vc);
@@ -507,12 +565,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // re-read the last block): a load that is issued on some paths only would force
   // the compiler to wait for *all* outstanding loads wherever it needs one of
   // them.
-  constexpr int CHG = Cfg::CHG;
-  // First chunk: the first step's weights (the longest latency) go out first,
-  // then the x copies, then the first scales; loads complete in order, so waiting
-  // for the x copies also waits for those weights, which step 0 needs anyway.
-  qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
-  x_chunk_load(0, min(CHG, steps_total));
+  // First chunk: weights of step 0 and the x copies are under way (issued at the top of the
+  // kernel); the first blockwise scales follow them.
   qmm_static_for<kBw>([&](auto tc) { bw_fetch(0, tc); });
   {
     // vmcnt(kInFlight): everything older than the first scales has landed
@@ -520,13 +574,16 @@ qmm_skinny_kernel(SkinnyArgs a) {
     __builtin_amdgcn_s_waitcnt(((kInFlight >> 4) << 14) | 0x0F70 | (kInFlight & 15));
   }
   qmm_lds_barrier();
+  fetch_channel_scales();  // (per-channel) needed at the very end: their latency hides behind the main loop
   int s0 = 0;  // this wave's next step
   for (int c0 = 0; c0 < steps_total; c0 += CHG) {
     const int nst = min(CHG, steps_total - c0);
     if (c0 > 0) {
       qmm_lds_barrier();                   // every wave has finished reading the old columns
-      x_chunk_load(c0, nst);
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+      if constexpr (kCopiers == 0) {
+        x_chunk_load(c0, 0, nst);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+      }
       qmm_lds_barrier();
     }
     int s_end = min(my_steps, (c0 + CHG) / KW);
@@ -535,22 +592,31 @@ qmm_skinny_kernel(SkinnyArgs a) {
     if constexpr (KW == 1 && P == 1) {
       if (c0 + CHG >= steps_total) --s_end;
     }
-    for (; s0 < s_end; s0 += P) {
-      qmm_static_for<P>([&](auto hc) {
-        const int s = s0 + hc;
-        const int gs = s * KW + kw;
-        // (a step past the end, which only occurs to complete a trip around the
-        // ring, has every sub-step beyond K: it issues its loads and computes nothing)
-        compute(hc, min(gs - c0, nst - 1), s, qmm_const<1>{});
-      });
+    auto run_steps = [&](int s_to) __attribute__((always_inline)) {
+      for (; s0 < s_to; s0 += P) {
+        qmm_static_for<P>([&](auto hc) {
+          const int s = s0 + hc;
+          const int gs = s * KW + kw;
+          // (a step past the end, which only occurs to complete a trip around the
+          // ring, has every sub-step beyond K: it issues its loads and computes nothing)
+          compute(hc, min(gs - c0, nst - 1), s, qmm_const<1>{});
+        });
+      }
+    };
+    if (c0 == 0 && second_meeting) {
+      // the steps whose columns were waited for (never a wave's last step: nst0 > kFirstTiles),
+      // then the meeting with the copying waves: the rest of the chunk's columns are there
+      run_steps(min(s_end, kFirstTiles / KW));
+      qmm_lds_barrier();
     }
+    run_steps(s_end);
     if constexpr (KW == 1 && P == 1) {
       if (c0 + CHG >= steps_total) compute(qmm_const<0>{}, s0 - c0, s0, qmm_const<0>{});
     }
   }
 
   // ---- reduction over k-splits, final rounding, store ------------------------------------
-  const int zpo_dt = qmm_promote(x_dt, a.zp_dt);
+  const int zpo_dt = qmm_promote(x_dt, zp_dt);
   if constexpr (KW > 1) {
     __syncthreads();  // every wave is done with the x tiles: reuse LDS
     float* red = (float*)smem;  // [KW][RW][slot][64]
@@ -600,16 +666,16 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const int m = 16 * mt + r;
     const int n = n_wave + 4 * g;
     if (m < M && n < N) {
-      float o0 = qmm_round_dt(sacc[mt][0], a.out_dt), o1 = qmm_round_dt(sacc[mt][1], a.out_dt);
-      float o2 = qmm_round_dt(sacc[mt][2], a.out_dt), o3 = qmm_round_dt(sacc[mt][3], a.out_dt);
+      float o0 = qmm_round_dt(sacc[mt][0], out_dt), o1 = qmm_round_dt(sacc[mt][1], out_dt);
+      float o2 = qmm_round_dt(sacc[mt][2], out_dt), o3 = qmm_round_dt(sacc[mt][3], out_dt);
       if constexpr (HASZP) {
-        o0 = qmm_round_dt(o0 - qmm_round_dt(zacc[mt][0], zpo_dt), a.out_dt);
-        o1 = qmm_round_dt(o1 - qmm_round_dt(zacc[mt][1], zpo_dt), a.out_dt);
-        o2 = qmm_round_dt(o2 - qmm_round_dt(zacc[mt][2], zpo_dt), a.out_dt);
-        o3 = qmm_round_dt(o3 - qmm_round_dt(zacc[mt][3], zpo_dt), a.out_dt);
+        o0 = qmm_round_dt(o0 - qmm_round_dt(zacc[mt][0], zpo_dt), out_dt);
+        o1 = qmm_round_dt(o1 - qmm_round_dt(zacc[mt][1], zpo_dt), out_dt);
+        o2 = qmm_round_dt(o2 - qmm_round_dt(zacc[mt][2], zpo_dt), out_dt);
+        o3 = qmm_round_dt(o3 - qmm_round_dt(zacc[mt][3], zpo_dt), out_dt);
       }
       // (a store dtype narrower than out_dt is the caller's final cast: one more rounding, done by the conversion)
-      const int st = a.store_dt;
+      const int st = store_dt;
       const size_t idx = (size_t)m * N + n;
       if ((N & 3) == 0) {  // 4 consecutive channels: one aligned 8- or 16-byte store
         if (st == XLA_AMD_DT_F32) {
@@ -632,27 +698,36 @@ qmm_skinny_kernel(SkinnyArgs a) {
   });
 }
 
-template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, int NW = kWaves, int WSEG = kWSeg>
+template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, bool UNI, int NW = kWaves, int WSEG = kWSeg>
 int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
   using Cfg = SkinnyCfg<XT, BITS, MT, KW, NW, WSEG>;
   if constexpr (!Cfg::kFits) {
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: tile does not fit in LDS");
   } else {
-    auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, NW, WSEG>;
+    auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, UNI, NW, WSEG>;
     static std::atomic<uint64_t> lds_set{0};
     const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(Cfg::CHG), lds_set, "weight_only_skinny hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
     const int steps = (a.K + Cfg::KS - 1) / Cfg::KS;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(NW * 64), Cfg::lds_bytes(steps), stream, a);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3((NW + skinny_copier_waves<MT, RED>()) * 64), Cfg::lds_bytes(steps), stream, a);
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
 
 template <int XT, int BITS, int MT, int KW, int RED>
 int launch_zp(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
-  return haszp ? launch_kernel<XT, BITS, MT, KW, RED, true>(a, stream)
-               : launch_kernel<XT, BITS, MT, KW, RED, false>(a, stream);
+  const bool uni = a.scale_dt == XT && a.zp_dt == XT && a.out_dt == XT && a.dot_dt == XT && a.store_dt == XT;
+  if (uni) {
+    return haszp ? launch_kernel<XT, BITS, MT, KW, RED, true, true>(a, stream)
+                 : launch_kernel<XT, BITS, MT, KW, RED, false, true>(a, stream);
+  }
+  if constexpr (RED == kRedRaw) {
+    return haszp ? launch_kernel<XT, BITS, MT, KW, RED, true, false>(a, stream)
+                 : launch_kernel<XT, BITS, MT, KW, RED, false, false>(a, stream);
+  } else {
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny: blockwise weights need scale, zero point and result of x's dtype");
+  }
 }
 
 // k-splits per workgroup: as few as keep >= ~200 workgroups, and only where the
