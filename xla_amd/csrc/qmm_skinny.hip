@@ -153,16 +153,23 @@ struct SkinnyCfg {
   static constexpr int NLD = 16 * WSEG / 1024;               // 1 KB weight loads per wave per step
   static constexpr int BLK = BITS == 8 ? 2048 : 1024;        // bytes of one (16 channels x 128 columns) weight block
   static constexpr int X_TILE = XROWS * XROW;                // the x columns of one step, all rows
-  static constexpr int CH = kLdsLimit / X_TILE;              // steps whose x columns are resident in LDS together
   // Steps of weight loads in flight per wave (register ring).  One step is
   // 8 KB per wave, 7 MB over the chip: enough to cover the memory latency; with
   // two or more the measured time goes *up* (the extra requests only queue).
   static constexpr int P = 1;
-  static constexpr int CHG = CH / (P * KW) * (P * KW);       // ... rounded so that a chunk holds whole trips around the ring for every wave
-  static constexpr bool kFits = CHG >= P * KW;
+  // x is resident in LDS a chunk of steps at a time.  A chunk holds whole trips around the
+  // ring for every wave (a multiple of P * KW steps).  With two chunk slots the next chunk is
+  // copied while the current one is used (CS2 steps per chunk); with one slot the workgroup
+  // stops while a chunk is replaced (CS1 steps per chunk).
+  static constexpr int CS1 = kLdsLimit / X_TILE / (P * KW) * (P * KW);
+  // (at most 4 steps per chunk with two slots: the first chunk is all that step 0 waits for)
+  static constexpr int CS2 = (kLdsLimit / (2 * X_TILE) < 4 ? kLdsLimit / (2 * X_TILE) : 4) / (P * KW) * (P * KW);
+  static constexpr bool kFits = CS1 >= P * KW;
   static constexpr int kRedBytes = NW * 16 * MT * 256;       // cross-wave reduction scratch (reuses the x tiles)
-  static constexpr int lds_bytes(int steps) {
-    const int x = (steps < CHG ? steps : CHG) * X_TILE;
+  static constexpr int lds_bytes(int steps, int slots) {
+    const int cs = slots == 2 ? CS2 : CS1;
+    const int tiles = steps <= cs ? steps : slots * cs;
+    const int x = tiles * X_TILE;
     return x > kRedBytes ? x : kRedBytes;
   }
   static_assert(WSEG == 512 || (WSEG == 256 && BITS == 8), "weight segment");
@@ -173,6 +180,11 @@ struct SkinnyCfg {
 // more (two x tiles with per-block scale accumulators) runs without them, and its computing
 // waves copy x themselves.
 template <int MT, int RED> constexpr int skinny_copier_waves() { return (MT == 2 && RED != 1 /*kRedRaw*/) ? 0 : 4; }
+// Chunk slots of x in LDS: two (the copying waves fill one while the other is used) when there
+// are copying waves and two chunks fit, else one.
+template <typename Cfg, int MT, int RED, int KW> constexpr int skinny_slots() {
+  return (skinny_copier_waves<MT, RED>() > 0 && Cfg::CS2 >= Cfg::P * KW) ? 2 : 1;
+}
 
 // UNI: scale, zero point, dot product, result and stored tensor all have x's dtype (the common
 // case, and the only one for blockwise weights): the dtypes are compile-time constants then, and
@@ -240,24 +252,28 @@ qmm_skinny_kernel(SkinnyArgs a) {
   auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {
     qmm_static_for<SUB>([&](auto tc) { load_sub(pc, s, tc); });
   };
-  // The x columns of global steps c0+t0 .. c0+t1-1 into the LDS tiles t0 .. t1-1.  The copying
-  // waves (the extra ones, or all waves when there are none) share the rows below M of every
-  // tile, a row per instruction (rows from
-  // M on are never stored, so their x is not copied: a decode step of one row copies
-  // 1/16 of a tile).  The loops are uniform and free of per-piece conditions: this code
-  // runs once per wave, straight after launch, and every branch in it costs an
-  // instruction fetch that nothing hides.
+  // x is used a chunk of CS steps at a time; chunk c lives in LDS slot c % kSlots (CS tiles
+  // per slot).  x_chunk_load copies chunk c: the copying waves (the extra ones, or all waves
+  // when there are none) share the rows below M of every tile, a row per instruction (rows
+  // from M on are never stored, so their x is not copied: a decode step of one row copies
+  // 1/16 of a tile).
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   const int x_rows = min(M, Cfg::XROWS);
   constexpr int kCopiers = skinny_copier_waves<MT, RED>();
+  constexpr int kSlots = skinny_slots<Cfg, MT, RED, KW>();
+  constexpr int CS = kSlots == 2 ? Cfg::CS2 : Cfg::CS1;
   constexpr int kCopyWaves = kCopiers > 0 ? kCopiers : NW;
   const int copy_wave = kCopiers > 0 ? wave - NW : wave;
-  auto x_chunk_load = [&](int c0, int t0, int t1) __attribute__((always_inline)) {
+  const int n_chunks = (steps_total + CS - 1) / CS;
+  auto x_chunk_load = [&](int c) __attribute__((always_inline)) {
+    const int c0 = c * CS;
+    const int nst = min(CS, steps_total - c0);
+    char* const slot = smem + (kSlots == 2 ? (c & 1) * (CS * X_TILE) : 0);
     for (int row = copy_wave; row < x_rows; row += kCopyWaves) {
       const char* xrow = x_base + (size_t)row * ((size_t)K * XB) + (size_t)c0 * XROW;  // row `row`, first column of the chunk
-      char* lrow = smem + row * XROW;
+      char* lrow = slot + row * XROW;
       const int sw = row & 15;
-      for (int t = t0; t < t1; ++t) {
+      for (int t = 0; t < nst; ++t) {
         const char* xp = xrow + (size_t)t * XROW;
         char* dst = lrow + t * X_TILE;
         if ((c0 + t + 1) * KS <= K) {
@@ -280,39 +296,34 @@ qmm_skinny_kernel(SkinnyArgs a) {
     }
   };
   // Copying all of x into every compute unit (the same 128 KB for each of them, out of a few L2
-  // slices) takes longer than the first weights take to arrive from memory, so only the x
-  // columns of the first kFirstTiles steps are waited for before step 0; the rest land while
-  // those steps run, and the workgroup meets once more before step kFirstTiles (a multiple
-  // of KW: every wave has the same number of steps before that).
+  // slices) takes longer than the first weights take to arrive from memory, so step 0 waits for
+  // the first chunk only; the next chunk lands while the current one is used, and the workgroup
+  // meets once per chunk.
   //
-  // The computing waves cannot do that themselves: with global -> LDS copies in flight when they
-  // enter the main loop, the compiler can no longer count their loads in flight and turns every
-  // wait of the loop into a wait for all of them.  So kCopiers extra waves do all the copying
-  // and nothing else: they wait for their copies, meet the workgroup at each of its meeting
-  // points, and leave.  The computing waves only request weights.
-  constexpr int CHG = Cfg::CHG;
-  constexpr int kFirstTiles = 4;  // (a multiple of every KW)
-  const int nst0 = min(CHG, steps_total);
-  const bool second_meeting = kCopiers > 0 && nst0 > kFirstTiles;  // uniform over the workgroup
+  // The computing waves cannot do the copying themselves: with global -> LDS copies in flight
+  // when they enter the main loop, the compiler can no longer count their loads in flight and
+  // turns every wait of the loop into a wait for all of them.  So kCopiers extra waves do all
+  // the copying and nothing else: they wait for their copies, meet the workgroup at each of
+  // its meeting points, and leave.  The computing waves only request weights.
   if constexpr (kCopiers > 0) {
     // (marked unlikely so that this block is laid out behind the computing waves' code: they
     // then run straight on from the kernel's entry to their first loads; a taken branch over
     // this block would cost them an instruction fetch from memory, the weights of the
     // previous launch having pushed the code out of L2)
     if (__builtin_expect(wave >= NW, 0)) {
-      for (int c0 = 0; c0 < steps_total; c0 += CHG) {
-        if (c0 > 0) qmm_bare_barrier();      // every wave has finished reading the old columns
-        const int nst = min(CHG, steps_total - c0);
-        if (c0 == 0 && second_meeting) {
-          x_chunk_load(0, 0, kFirstTiles);
-          __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
-          qmm_bare_barrier();
-          x_chunk_load(0, kFirstTiles, nst);
-        } else {
-          x_chunk_load(c0, 0, nst);
+      x_chunk_load(0);
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+      for (int c = 0; c < n_chunks; ++c) {
+        if (kSlots == 1 && c > 0) {
+          qmm_bare_barrier();  // every wave has finished reading the old columns
+          x_chunk_load(c);
+          __builtin_amdgcn_s_waitcnt(0x0F70);
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        qmm_bare_barrier();
+        qmm_bare_barrier();    // chunk c is there (and, with two slots, chunk c - 1 has been read)
+        if (kSlots == 2 && c + 1 < n_chunks) {
+          x_chunk_load(c + 1);
+          __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
       }
       if constexpr (KW > 1) { qmm_bare_barrier(); qmm_bare_barrier(); }  // the two of the k-split reduction
       return;
@@ -326,7 +337,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   if constexpr (kCopiers == 0) {
     // Loads complete in order, so waiting for the copies also waits for those weights, which
     // step 0 needs anyway.
-    x_chunk_load(0, 0, nst0);
+    x_chunk_load(0);
     __builtin_amdgcn_sched_barrier(0);
   }
 
@@ -552,66 +563,60 @@ qmm_skinny_kernel(SkinnyArgs a) {
   };
 
   // ---- main loop ---------------------------------------------------------------------
-  // The x columns of a chunk of up to CHG steps are resident in LDS; the workgroup
-  // meets only when they are replaced, and between those points every wave runs
-  // its steps at its own pace (wait for its weights, multiply), so that the
-  // waves of a compute unit drift apart and their memory waits, LDS traffic and
-  // arithmetic overlap.
-  // Every wave runs the chunk loop the same number of times, whether it has
-  // steps in a chunk or not: the barriers always match.  A chunk holds whole
-  // trips around the ring for every wave, so each chunk starts on ring slot 0.
+  // The x columns of a chunk of CS steps are resident in LDS; the workgroup meets once per
+  // chunk, and between those points every wave runs its steps at its own pace (wait for its
+  // weights, multiply), so that the waves of a compute unit drift apart and their memory
+  // waits, LDS traffic and arithmetic overlap.
+  // Every wave runs the chunk loop the same number of times, whether it has steps in a chunk
+  // or not: the barriers always match.  A chunk holds whole trips around the ring for every
+  // wave, so each chunk starts on ring slot 0.
   //
   // Weight loads are issued unconditionally, also for steps past the end (those
   // re-read the last block): a load that is issued on some paths only would force
   // the compiler to wait for *all* outstanding loads wherever it needs one of
   // them.
-  // First chunk: weights of step 0 and the x copies are under way (issued at the top of the
-  // kernel); the first blockwise scales follow them.
+  // First chunk: weights of step 0 are under way (issued at the top of the kernel) and so
+  // are the x copies; the first blockwise scales follow them.
   qmm_static_for<kBw>([&](auto tc) { bw_fetch(0, tc); });
   {
     // vmcnt(kInFlight): everything older than the first scales has landed
     constexpr int kInFlight = RED != kRedRaw ? (HASZP ? 2 : 1) * kBw : 0;
     __builtin_amdgcn_s_waitcnt(((kInFlight >> 4) << 14) | 0x0F70 | (kInFlight & 15));
   }
-  qmm_lds_barrier();
+  qmm_bare_barrier();
   fetch_channel_scales();  // (per-channel) needed at the very end: their latency hides behind the main loop
   int s0 = 0;  // this wave's next step
-  for (int c0 = 0; c0 < steps_total; c0 += CHG) {
-    const int nst = min(CHG, steps_total - c0);
-    if (c0 > 0) {
-      qmm_lds_barrier();                   // every wave has finished reading the old columns
-      if constexpr (kCopiers == 0) {
-        x_chunk_load(c0, 0, nst);
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+  for (int c = 0; c < n_chunks; ++c) {
+    const int c0 = c * CS;
+    const int nst = min(CS, steps_total - c0);
+    const int tile0 = kSlots == 2 ? (c & 1) * CS : 0;
+    if (c > 0) {
+      if constexpr (kSlots == 1) {
+        qmm_bare_barrier();                    // every wave has finished reading the old columns
+        if constexpr (kCopiers == 0) {
+          x_chunk_load(c);
+          __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+        }
       }
-      qmm_lds_barrier();
+      qmm_bare_barrier();                      // chunk c is there
     }
-    int s_end = min(my_steps, (c0 + CHG) / KW);
+    int s_end = min(my_steps, (c0 + CS) / KW);
     // Without k-splits the wave's last step lies in the last chunk: it is run
     // after the loop, in a form that fetches nothing more.
     if constexpr (KW == 1 && P == 1) {
-      if (c0 + CHG >= steps_total) --s_end;
+      if (c + 1 == n_chunks) --s_end;
     }
-    auto run_steps = [&](int s_to) __attribute__((always_inline)) {
-      for (; s0 < s_to; s0 += P) {
-        qmm_static_for<P>([&](auto hc) {
-          const int s = s0 + hc;
-          const int gs = s * KW + kw;
-          // (a step past the end, which only occurs to complete a trip around the
-          // ring, has every sub-step beyond K: it issues its loads and computes nothing)
-          compute(hc, min(gs - c0, nst - 1), s, qmm_const<1>{});
-        });
-      }
-    };
-    if (c0 == 0 && second_meeting) {
-      // the steps whose columns were waited for (never a wave's last step: nst0 > kFirstTiles),
-      // then the meeting with the copying waves: the rest of the chunk's columns are there
-      run_steps(min(s_end, kFirstTiles / KW));
-      qmm_lds_barrier();
+    for (; s0 < s_end; s0 += P) {
+      qmm_static_for<P>([&](auto hc) {
+        const int s = s0 + hc;
+        const int gs = s * KW + kw;
+        // (a step past the end, which only occurs to complete a trip around the
+        // ring, has every sub-step beyond K: it issues its loads and computes nothing)
+        compute(hc, tile0 + min(gs - c0, nst - 1), s, qmm_const<1>{});
+      });
     }
-    run_steps(s_end);
     if constexpr (KW == 1 && P == 1) {
-      if (c0 + CHG >= steps_total) compute(qmm_const<0>{}, s0 - c0, s0, qmm_const<0>{});
+      if (c + 1 == n_chunks) compute(qmm_const<0>{}, tile0 + s0 - c0, s0, qmm_const<0>{});
     }
   }
 
@@ -706,11 +711,12 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
   } else {
     auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, UNI, NW, WSEG>;
     static std::atomic<uint64_t> lds_set{0};
-    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(Cfg::CHG), lds_set, "weight_only_skinny hipFuncSetAttribute");
+    constexpr int kSlots = skinny_slots<Cfg, MT, RED, KW>();
+    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20, kSlots), lds_set, "weight_only_skinny hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
     const int steps = (a.K + Cfg::KS - 1) / Cfg::KS;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3((NW + skinny_copier_waves<MT, RED>()) * 64), Cfg::lds_bytes(steps), stream, a);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3((NW + skinny_copier_waves<MT, RED>()) * 64), Cfg::lds_bytes(steps, kSlots), stream, a);
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
