@@ -65,6 +65,7 @@ extern "C" {
 #define XLA_AMD_KERNEL_SKINNY_MFMA 1 /* weight-streaming GEMV / skinny GEMM       */
 #define XLA_AMD_KERNEL_W8A8_MFMA 2  /* LDS-tiled int8 MFMA GEMM                   */
 #define XLA_AMD_KERNEL_W8A8_GENERIC 3
+#define XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM 4 /* tiled bf16/f16 MFMA GEMM on int8 weights */
 
 int xla_amd_qmm_abi_version(void);
 
@@ -153,6 +154,35 @@ int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const voi
                                    const void* zp, void* out, int64_t M, int64_t N, int64_t K,
                                    int64_t C, int bits, int x_dt, int scale_dt, int zp_dt,
                                    int dot_dt, int out_dt, int store_dt, void* stream);
+
+/*
+ * Bytes of workspace xla_amd_qmm_weight_only_gemm needs for a shape (0 when it
+ * needs none, or for arguments it rejects).
+ */
+size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Weight-only quantized matmul for many rows of x (prefill-sized M), and for
+ * few output channels with a long K: a tiled MFMA GEMM that reads the weight
+ * once per tile of up to 128 rows, where xla_amd_qmm_weight_only_skinny reads
+ * it once per 32 rows.  Replaces the same reference statements with the same
+ * rounding points,
+ *   out = F.linear(x, w) * scaler;  out -= rowsum(x) (x) zp   (xla_quantized_matmul.py:113-114, :125-133)
+ * and, with dot_dt = f32, the float branch of the Pallas kernel
+ * (pallas_kernels/quantized_matmul_kernel.py:108-121).
+ * Per-channel int8 weights only (w_tiled from xla_amd_qmm_tile_weight with
+ * bits == 8), x [M,K] bf16 or f16, K % 128 == 0; other cases return
+ * XLA_AMD_QMM_EUNSUPPORTED (the streaming kernel takes them).  dtype arguments
+ * as for xla_amd_qmm_weight_only_skinny.  When K is split over workgroups the
+ * partial sums live in `workspace` (device memory of at least
+ * xla_amd_qmm_weight_only_gemm_workspace_bytes(M, N, K) bytes, 16-byte
+ * aligned, free again when the call's work has completed); it may be NULL
+ * when that size is 0.
+ */
+int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, const void* scale, const void* zp,
+                                 void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                                 int64_t K, int x_dt, int scale_dt, int zp_dt, int dot_dt, int out_dt,
+                                 int store_dt, void* stream);
 
 /*
  * Weight-only quantized matmul for any shape, reading the operator's own

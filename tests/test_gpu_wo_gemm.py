@@ -1,0 +1,94 @@
+"""GPU parity of the weight-only tiled GEMM (many rows of x, or few channels with a long K) against the CPU oracle."""
+import pytest
+import torch
+
+from tests import cases
+from oracle import quantized_matmul_oracle as oracle
+from xla_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+  import xla_amd.experimental.custom_kernel  # noqa: F401
+  import xla_amd.experimental.xla_quantized_matmul as qmm
+  return qmm
+
+
+def check(actual, expected, what=""):
+  assert actual.dtype == expected.dtype, f"{what}: dtype {actual.dtype} vs {expected.dtype}"
+  assert actual.shape == expected.shape
+  a = actual.cpu()
+  assert torch.isfinite(a.float()).all(), what
+  rl2 = cases.rel_l2(a, expected)
+  assert cases.within_tolerance(a, expected), f"{what}: rel-L2 {rl2:.3e} outside tolerance"
+  return rl2
+
+
+def wo_gemm(ops, x, w, s, z, dot_dtype=None, store_dtype=None):
+  """Calls xla_amd_qmm_weight_only_gemm directly (whatever the dispatcher would choose)."""
+  lib = _lib.load()
+  m, k = x.shape
+  n = w.shape[0]
+  wt = ops._tiled_weight(w, 8, _lib.W_NK)
+  out_dtype = torch.promote_types(x.dtype, s.dtype)
+  store_dtype = store_dtype or out_dtype
+  out = torch.empty(m, n, dtype=store_dtype, device=x.device)
+  nbytes = lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k)
+  ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+  zp_dt = _lib.dt(z.dtype) if z is not None else _lib.dt(x.dtype)
+  rc = lib.xla_amd_qmm_weight_only_gemm(x.data_ptr(), wt.data_ptr(), s.data_ptr(), _lib.ptr(z), out.data_ptr(), ws.data_ptr(),
+                                        nbytes, m, n, k, _lib.dt(x.dtype), _lib.dt(s.dtype), zp_dt,
+                                        _lib.dt(dot_dtype or x.dtype), _lib.dt(out_dtype), _lib.dt(store_dtype),
+                                        torch.cuda.current_stream().cuda_stream)
+  _lib.check(rc, "weight_only_gemm")
+  return out
+
+
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("zp", [False, True])
+def test_wo_gemm_shapes(ops, xdt, zp):
+  # every row-tile height (32 / 64 / 128 rows), both tile widths, with and without a K split, M / N tails,
+  # one to many K steps, several chunks of x
+  for (m, n, k) in [(33, 256, 512), (64, 100, 1024), (17, 4096, 14336), (32, 1024, 4096), (128, 512, 128), (200, 333, 2560),
+                    (300, 700, 1024), (48, 64, 8192), (2, 16, 128), (130, 2048, 2048)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)
+    z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(xdt) if zp else None
+    exp = oracle.quantized_matmul(x, w, s, z)
+    out = wo_gemm(ops, x.cuda(), w.cuda(), s.cuda(), None if z is None else z.cuda())
+    rl2 = check(out, exp, f"wo_gemm {m, n, k, xdt, zp}")
+    assert rl2 < 1e-3, (m, n, k, rl2)
+
+
+def test_wo_gemm_mixed_dtypes_and_float_branch(ops):
+  x, w, s, _ = cases.per_channel_int8(100, 384, 1024, torch.bfloat16, torch.float32, seed=3)
+  z = torch.randn(384, generator=cases.gen(6)) * 0.01
+  out = wo_gemm(ops, x.cuda(), w.cuda(), s.cuda(), z.cuda())
+  assert out.dtype == torch.float32
+  check(out, oracle.quantized_matmul(x, w, s, z), "bf16 x, f32 scale / zp")
+  # the dedicated kernel's float branch: f32 accumulation, f32 scale, one cast
+  out = wo_gemm(ops, x.cuda(), w.cuda(), s.cuda(), None, dot_dtype=torch.float32, store_dtype=torch.bfloat16)
+  rl2 = check(out, oracle.quantized_matmul_int8(x, w, s), "float branch")
+  assert rl2 < 3e-4
+
+
+def test_weight_only_prefill_through_the_operator(ops):
+  # cfg2's shape with a prefill-sized M: the operator takes the tiled GEMM above 32 rows
+  m, n, k = 2048, 14336, 4096
+  x, w, s, _ = cases.per_channel_int8(m, n, k, torch.bfloat16, torch.bfloat16, seed=2)
+  before = ops.counters["wo_gemm"]
+  out = torch.ops.xla.quantized_matmul(x.cuda(), w.cuda(), s.cuda())
+  assert ops.counters["wo_gemm"] == before + 1
+  rows = torch.arange(0, m, 29)
+  rl2 = check(out[rows.cuda()], oracle.quantized_matmul(x[rows], w, s), "weight-only prefill rows")
+  assert rl2 < 5e-4
+  # size-independent: a row of the result depends on that row of x only
+  out2 = torch.ops.xla.quantized_matmul(x[rows].cuda(), w.cuda(), s.cuda())
+  assert cases.rel_l2(out2.cpu(), out[rows.cuda()].cpu()) < 1e-3
+  # the module and 3-D activations take the same route
+  from xla_amd.experimental.xla_quantized_matmul import XlaQuantizedLinear
+  lin = XlaQuantizedLinear(k, n, is_symmetric=True)
+  lin.load_quantized_weight(w.cuda(), s.cuda())
+  x3 = x[:96].reshape(2, 48, k)
+  check(lin(x3.cuda()), oracle.quantized_matmul(x3, w, s), "module, 3-D x")

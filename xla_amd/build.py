@@ -16,16 +16,22 @@ OBJ_DIR = os.path.join(PKG_DIR, "csrc", "build")
 LIB_PATH = os.path.join(PKG_DIR, "libxla_amd_qmm.so")
 
 # (source, extra flags, object name); the skinny kernels are built once per
-# activation dtype so that the three units compile in parallel
+# activation dtype and the weight-only GEMM once per (dtype, row tile) so that
+# the units compile in parallel
 SOURCES = [
-    ("qmm_api.hip", [], "qmm_api.o"),
-    ("qmm_generic.hip", [], "qmm_generic.o"),
-    ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=0"], "qmm_skinny_f32.o"),
+    # the slow units first: eight compilers run at a time
+    ("qmm_wo_gemm.hip", ["-DQMM_WO_XT=1", "-DQMM_WO_MT=8"], "qmm_wo_gemm_bf16_mt8.o"),
+    ("qmm_wo_gemm.hip", ["-DQMM_WO_XT=2", "-DQMM_WO_MT=8"], "qmm_wo_gemm_f16_mt8.o"),
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=1"], "qmm_skinny_bf16.o"),
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=2"], "qmm_skinny_f16.o"),
+    ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=0"], "qmm_skinny_f32.o"),
+    ("qmm_wo_gemm.hip", ["-DQMM_WO_XT=1", "-DQMM_WO_MT=4"], "qmm_wo_gemm_bf16_mt4.o"),
+    ("qmm_wo_gemm.hip", ["-DQMM_WO_XT=2", "-DQMM_WO_MT=4"], "qmm_wo_gemm_f16_mt4.o"),
+    ("qmm_w8a8_gemm.hip", [], "qmm_w8a8_gemm.o"),
+    ("qmm_api.hip", [], "qmm_api.o"),
+    ("qmm_generic.hip", [], "qmm_generic.o"),
     ("qmm_quant_act.hip", [], "qmm_quant_act.o"),
     ("qmm_qdq.hip", [], "qmm_qdq.o"),
-    ("qmm_w8a8_gemm.hip", [], "qmm_w8a8_gemm.o"),
     ("qmm_linear.hip", [], "qmm_linear.o"),
 ]
 

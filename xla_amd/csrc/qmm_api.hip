@@ -56,12 +56,14 @@ extern "C" size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits) {
 extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, int bits,
                                     int x_dt, int quantize_activation) {
   (void)N;
-  (void)x_dt;
   if (quantize_activation) {
     if (K % 64 == 0 && M * N >= 64 * 64) return XLA_AMD_KERNEL_W8A8_MFMA;
     return XLA_AMD_KERNEL_W8A8_GENERIC;
   }
   if (C <= 0) C = K;
+  // many rows of 2-byte x against per-channel int8 weights: the tiled GEMM reads the weight once
+  // per 128 rows, the streaming kernel once per 32
+  if (C == K && bits == 8 && K % 128 == 0 && x_dt != XLA_AMD_DT_F32 && M > 32) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
   if (K % 128 == 0 && C % 128 == 0 && (bits == 8 || bits == 4) && M >= 1 &&
       (C == K || (N % 4 == 0 && (K / C) * N >= 8)))  // blockwise: vector loads of 4 channels' scales
     return XLA_AMD_KERNEL_SKINNY_MFMA;

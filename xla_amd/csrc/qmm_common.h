@@ -68,12 +68,21 @@ __device__ __forceinline__ float qmm_bf16_to_f32(uint16_t b) {
   return __uint_as_float(((uint32_t)b) << 16);
 }
 
-// Round-to-nearest-even f32 -> bf16 bit pattern (NaN stays NaN).
+// Round-to-nearest-even f32 -> bf16 bit pattern (NaN stays NaN): the hardware conversion
+// (v_cvt_pk_bf16_f32).
 __device__ __forceinline__ uint16_t qmm_f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+// Two values at once, lo in the low half.
+__device__ __forceinline__ uint32_t qmm_f32x2_to_bf16x2(float lo, float hi) {
+  typedef float qmm_f32x2_t __attribute__((ext_vector_type(2)));
+  typedef __bf16 qmm_bf16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(qmm_f32x2_t{lo, hi}, qmm_bf16x2_t));
+}
+__device__ __forceinline__ uint32_t qmm_f32x2_to_f16x2(float lo, float hi) {
+  typedef float qmm_f32x2_t __attribute__((ext_vector_type(2)));
+  typedef _Float16 qmm_f16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(qmm_f32x2_t{lo, hi}, qmm_f16x2_t));
 }
 
 __device__ __forceinline__ float qmm_f16_to_f32(uint16_t h) {

@@ -1,0 +1,584 @@
+// Weight-only quantized matmul for many rows of x: a tiled bf16/f16 MFMA GEMM whose B
+// operand is the int8 weight, converted to x's dtype in registers (exact).
+//
+// The weight-streaming kernel (qmm_skinny.hip) keeps up to 32 rows of x per pass and
+// re-reads the whole weight for every further 32 rows; its workgroups also each copy all
+// of x, which for a long K and few output channels is several times the weight itself.
+// This kernel covers those cases: a workgroup owns a tile of 16*MT rows x 64*NG channels,
+// every weight fragment is used against all row tiles from registers, and K can be split
+// over workgroups (each then copies only its slice of x); the partial sums of a split
+// go to a workspace and a second kernel adds them in a fixed order and finishes them.
+//
+// Operands.  Weights come from the tiled copy (xla_amd_qmm_tile_weight): one 2 KB block per
+// 16 channels x 128 columns, already in MFMA operand order, so a wave loads its fragments
+// straight into registers: no LDS traffic and no transposition for weights.  x goes through
+// LDS: the workgroup's rows, a chunk of K steps (128 columns each) at a time, in two chunk
+// slots; four extra waves do nothing but copy the next chunk (global -> LDS without
+// registers) while the four computing waves use the current one, and the workgroup meets
+// once per chunk.  (The computing waves must not issue such copies themselves: with copies
+// in flight the compiler can no longer count their register loads in flight and turns every
+// wait of the loop into a wait for all of them.)
+//
+// MFMA mapping (v_mfma_f32_16x16x32_bf16/f16, A = weights, B = x^T), as in the streaming
+// kernel: lane l is (r = l%16, g = l/16); for a block of 128 columns the lane supplies, for
+// weight channel r and for x row r of each 16-row tile, the columns 32g..32g+31 as four
+// instructions of 8 columns each.  D[i][j] lands in lane (j + 16*(i/4)), register i%4:
+// channel 4g + v, x row r: four consecutive channels of one row per lane.
+//
+// Arithmetic: the reference's per-channel sequence with its rounding points
+//   p = round_dot(sum_k x*w); out = round_out(scale * p);
+//   zero point: out = round_out(out - round_zpo(round_x(sum_k x) * zp)); stored as store_dt.
+//
+// This file is compiled once per (activation dtype, row tile) pair (-DQMM_WO_XT=1|2 for bf16 | f16,
+// -DQMM_WO_MT=4|8) so that the units build in parallel; the unit of bf16 with MT = 8 also
+// holds the second kernel of a K split and the C entry points.
+#include "qmm_common.h"
+
+#if !defined(QMM_WO_XT) || !defined(QMM_WO_MT)
+#error "compile with -DQMM_WO_XT=<XLA_AMD_DT_BF16|XLA_AMD_DT_F16 value> -DQMM_WO_MT=<4|8>"
+#endif
+
+struct WoGemmArgs {
+  const void* x;       // [M, K]
+  const uint8_t* w;    // tiled weight, 8 bits
+  const void* scale;   // [N]
+  const void* zp;      // [N] or null
+  void* out;           // [M, N] of store_dt (split == 1)
+  float* part;         // [split][M][N] partial dot products (split > 1)
+  float* part_xs;      // [split][M] partial row sums of x (split > 1, zero point)
+  int M, N, K;
+  int k_per_split;     // columns per K slice (a multiple of 128)
+  int split;
+  int scale_dt, zp_dt, dot_dt, out_dt, store_dt;
+};
+
+// one launcher per unit: row tile of 16 * MT rows, ng = 2 or 4 channel groups per computing wave
+int qmm_wo_launch_bf16_mt4(const WoGemmArgs& a, int ng, hipStream_t stream);
+int qmm_wo_launch_bf16_mt8(const WoGemmArgs& a, int ng, hipStream_t stream);
+int qmm_wo_launch_f16_mt4(const WoGemmArgs& a, int ng, hipStream_t stream);
+int qmm_wo_launch_f16_mt8(const WoGemmArgs& a, int ng, hipStream_t stream);
+
+namespace {
+
+constexpr int kComputeWaves = 4;
+constexpr int kCopyWaves = 4;
+constexpr int kLds = 160 * 1024;
+
+__device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
+  // {bf16(lo), bf16(hi)} by truncation: exact for integers of magnitude <= 256.
+  return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 v = __builtin_bit_cast(h2, __builtin_amdgcn_cvt_pkrtz(lo, hi));  // exact for small integers
+  return __builtin_bit_cast(uint32_t, v);
+}
+// 8 int8 weights (two dwords) -> 8 elements of the x dtype.
+template <int XT>
+__device__ __forceinline__ i32x4 cvt_w8(uint32_t d0, uint32_t d1) {
+  float f[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[i] = (float)(int8_t)(d0 >> (8 * i));
+    f[4 + i] = (float)(int8_t)(d1 >> (8 * i));
+  }
+  i32x4 o;
+  if constexpr (XT == XLA_AMD_DT_BF16) {
+    o[0] = pack_hi16(f[0], f[1]); o[1] = pack_hi16(f[2], f[3]);
+    o[2] = pack_hi16(f[4], f[5]); o[3] = pack_hi16(f[6], f[7]);
+  } else {
+    o[0] = pack_f16(f[0], f[1]); o[1] = pack_f16(f[2], f[3]);
+    o[2] = pack_f16(f[4], f[5]); o[3] = pack_f16(f[6], f[7]);
+  }
+  return o;
+}
+template <int XT>
+__device__ __forceinline__ f32x4 mfma16(i32x4 a, i32x4 b, f32x4 c) {
+  if constexpr (XT == XLA_AMD_DT_BF16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+}
+template <int XT> __device__ __forceinline__ i32x4 ones_frag() {
+  const uint32_t one2 = XT == XLA_AMD_DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
+  return i32x4{(int)one2, (int)one2, (int)one2, (int)one2};
+}
+
+template <int MT> struct WoCfg {
+  static constexpr int BM = 16 * MT;
+  static constexpr int X_TILE = BM * 256;                      // bytes of the x columns of one step (128 columns, 2-byte x)
+  static constexpr int kFit = kLds / (2 * X_TILE);             // steps per chunk slot that fit twice
+  static constexpr int CS = kFit < 8 ? kFit : 8;               // steps per chunk
+  static_assert(CS >= 1, "two chunk slots must fit in LDS");
+  static constexpr int lds_bytes(int steps) { return (steps <= CS ? steps : 2 * CS) * X_TILE; }
+};
+
+// The dtypes of the epilogue: those of the call, or (UNI) all equal to x's dtype and known at
+// compile time, which is the common case and removes every branch on a dtype.
+template <int XT, bool UNI> struct WoDts {
+  int scale_dt, zp_dt, dot_dt, out_dt, store_dt;
+  __device__ __forceinline__ explicit WoDts(const WoGemmArgs& a)
+      : scale_dt(UNI ? XT : a.scale_dt), zp_dt(UNI ? XT : a.zp_dt), dot_dt(UNI ? XT : a.dot_dt),
+        out_dt(UNI ? XT : a.out_dt), store_dt(UNI ? XT : a.store_dt) {}
+};
+
+// Scale (or zero point) of four consecutive channels as raw bits; channels past N repeat the last one.
+__device__ __forceinline__ void wo_load4_raw(const void* p, int n, int N, int dt, uint32_t raw[4]) {
+#pragma unroll
+  for (int v = 0; v < 4; ++v) raw[v] = qmm_load_raw(p, min(n + v, N - 1), dt);
+}
+
+// The reference's epilogue for four consecutive channels of one row:
+//   p = round_dot(dot); r = round_out(scale * p); with a zero point r = round_out(r - round_zpo(round_x(xsum) * zp)).
+template <class Dts>
+__device__ __forceinline__ void wo_finish4(const Dts& d, const uint32_t sraw[4], const uint32_t zraw[4], bool has_zp,
+                                           f32x4 dot, float xsum, int x_dt, float o[4]) {
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const float p = qmm_round_dt(dot[v], d.dot_dt);
+    float r = qmm_round_dt(qmm_from_raw(sraw[v], d.scale_dt) * p, d.out_dt);
+    if (has_zp) {
+      const int zpo_dt = qmm_promote(x_dt, d.zp_dt);
+      const float z = qmm_round_dt(qmm_round_dt(xsum, x_dt) * qmm_from_raw(zraw[v], d.zp_dt), zpo_dt);
+      r = qmm_round_dt(r - z, d.out_dt);
+    }
+    o[v] = r;
+  }
+}
+
+// Stores four consecutive channels of row m starting at channel n (n % 4 == 0).  VEC: N is a
+// multiple of 4, so the four channels exist and their address is aligned for one store.
+template <bool VEC>
+__device__ __forceinline__ void wo_store4(void* out, int m, int n, int N, const float o[4], int store_dt) {
+  const size_t idx = (size_t)m * N + n;
+  if constexpr (VEC) {
+    if (store_dt == XLA_AMD_DT_F32) {
+      *(f32x4*)((float*)out + idx) = f32x4{o[0], o[1], o[2], o[3]};
+    } else {
+      const bool bf = store_dt == XLA_AMD_DT_BF16;
+      const uint32_t lo = bf ? qmm_f32x2_to_bf16x2(o[0], o[1]) : qmm_f32x2_to_f16x2(o[0], o[1]);
+      const uint32_t hi = bf ? qmm_f32x2_to_bf16x2(o[2], o[3]) : qmm_f32x2_to_f16x2(o[2], o[3]);
+      *(i32x2*)((uint16_t*)out + idx) = i32x2{(int)lo, (int)hi};
+    }
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (n + v < N) qmm_store(out, idx + v, o[v], store_dt);
+  }
+}
+
+// The same epilogue and store when every dtype is bf16 and there is no zero point: two
+// values per conversion, and the rounded product is already the stored bit pattern.
+__device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, int N, const uint32_t sraw[4], f32x4 dot) {
+  uint32_t res[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint32_t p = qmm_f32x2_to_bf16x2(dot[2 * h], dot[2 * h + 1]);
+    const float p0 = __uint_as_float(p << 16), p1 = __uint_as_float(p & 0xffff0000u);
+    res[h] = qmm_f32x2_to_bf16x2(__uint_as_float(sraw[2 * h] << 16) * p0, __uint_as_float(sraw[2 * h + 1] << 16) * p1);
+  }
+  *(i32x2*)((uint16_t*)out + (size_t)m * N + n) = i32x2{(int)res[0], (int)res[1]};
+}
+
+// One unit of work: a tile of rows x channels over one K slice.
+struct WoItem {
+  int m0, n0, ks, k_begin, steps, n_chunks, rows;
+};
+
+// The kernel is persistent: workgroup b takes the work items b, b + gridDim.x, ... one after the
+// other.  The chunk ring simply runs on across items, so the copying waves fetch the first
+// chunk of the next item while the computing waves finish and store the current one, and the
+// computing waves request the next item's first weights before they store.
+template <int XT, int MT, int NG, bool HASZP, bool UNI>
+__global__ void __launch_bounds__((kComputeWaves + kCopyWaves) * 64)
+qmm_wo_gemm_kernel(WoGemmArgs a) {
+  using Cfg = WoCfg<MT>;
+  constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE, CS = Cfg::CS;
+  constexpr int BN = 64 * NG;  // channels per workgroup: NG groups of 16 per computing wave
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, g = lane >> 4;
+  const int M = a.M, N = a.N, K = a.K;
+  const int tiles_n = (N + BN - 1) / BN;
+  const int tiles = tiles_n * ((M + BM - 1) / BM);
+  const int n_items = tiles * a.split;
+  // item -> (K slice, row tile, column tile), column tiles fastest: workgroups that run together share x rows
+  auto item_of = [&](int it) __attribute__((always_inline)) {
+    WoItem w;
+    const int tile = it % tiles;
+    w.ks = it / tiles;
+    w.m0 = (tile / tiles_n) * BM;
+    w.n0 = (tile % tiles_n) * BN;
+    w.k_begin = w.ks * a.k_per_split;
+    w.steps = (min(K, w.k_begin + a.k_per_split) - w.k_begin) / 128;  // >= 1
+    w.n_chunks = (w.steps + CS - 1) / CS;
+    w.rows = min(BM, M - w.m0);  // live rows of this tile
+    return w;
+  };
+
+  if (__builtin_expect(wave >= kComputeWaves, 0)) {
+    // ---- copying waves: chunk after chunk of x into the two slots in turn, rows shared among them ----
+    const int cw = wave - kComputeWaves;
+    auto chunk_load = [&](const WoItem& w, int c, int slot_i) __attribute__((always_inline)) {
+      const int s0 = c * CS;
+      const int nst = min(CS, w.steps - s0);
+      char* const slot = smem + slot_i * (CS * X_TILE);
+      const char* const xb = (const char*)a.x + ((size_t)w.m0 * K + w.k_begin) * 2;
+      // a row of one step is 256 bytes: an instruction copies four consecutive rows
+      // (lane l: row l/16 of the four, chunk l%16), swizzled on the source side
+      for (int r4 = cw * 4; r4 < w.rows; r4 += kCopyWaves * 4) {
+        const int row = min(r4 + (lane >> 4), w.rows - 1);  // rows past the end repeat the last one
+        const int chunk = (lane & 15) ^ (row & 15);
+        const char* src = xb + (size_t)row * ((size_t)K * 2) + (size_t)s0 * 256 + chunk * 16;
+        char* dst = slot + r4 * 256;
+        for (int t = 0; t < nst; ++t)
+          __builtin_amdgcn_global_load_lds((const void*)(src + t * 256), (lds_ptr_t)(dst + t * X_TILE), 16, 0, 0);
+      }
+    };
+    int it = blockIdx.x;
+    WoItem cur = item_of(it);
+    int c = 0, ring = 0;  // ring: chunks since the kernel began; chunk `ring` lives in slot ring % 2
+    chunk_load(cur, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    for (;;) {
+      qmm_bare_barrier();  // chunk `ring` is there, chunk ring - 1 has been read
+      ++c; ++ring;
+      if (c == cur.n_chunks) {
+        it += gridDim.x;
+        if (it >= n_items) break;
+        cur = item_of(it);
+        c = 0;
+      }
+      chunk_load(cur, c, ring & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    return;
+  }
+
+  // ---- computing waves ----
+  // wave w owns the channel groups (n0/16 + w*NG) .. + NG-1 of the item's column tile
+  const int n_blk = K / 128;  // blocks per channel group in the tiled weight
+  const int groups = (N + 15) / 16;
+  const uint8_t* wp[NG];
+  i32x4 wreg[NG][2];
+  auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
+    qmm_static_for<NG>([&](auto gc) {
+      constexpr int gi = gc;
+      const int grp = min(w.n0 / 16 + wave * NG + gi, groups - 1);  // groups past N re-read the last one
+      wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * 2048 + lane * 16;
+    });
+  };
+  auto load_step = [&](int blk, auto hc) __attribute__((always_inline)) {
+    constexpr int h = hc;
+    qmm_static_for<NG>([&](auto gc) {
+      constexpr int gi = gc;
+      wreg[gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * 2048 + h * 1024));
+    });
+  };
+
+  f32x4 acc[NG][MT], xs[MT];
+  // one step (128 columns) out of LDS tile `tile`; the weight registers are refilled with
+  // block `next` as soon as each half has been used
+  auto compute = [&](int tile, int next, auto refillc) __attribute__((always_inline)) {
+    constexpr bool kRefill = refillc != 0;
+    const char* xbase = smem + tile * X_TILE;
+    qmm_static_for<4>([&](auto jc) {
+      constexpr int j = jc;
+      i32x4 xq[MT];
+      qmm_static_for<MT>([&](auto mc) {
+        constexpr int mt = mc;
+        xq[mt] = *(const i32x4*)(xbase + (16 * mt + r) * 256 + (((4 * g + j) ^ r) * 16));
+      });
+      qmm_static_for<NG>([&](auto gc) {
+        constexpr int gi = gc;
+        const i32x4 src = wreg[gi][j >> 1];
+        const i32x4 af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          acc[gi][mt] = mfma16<XT>(af, xq[mt], acc[gi][mt]);
+        });
+      });
+      if constexpr (HASZP) {
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt], xs[mt]);
+        });
+      }
+      if constexpr (kRefill && (j & 1)) load_step(next, qmm_const<(j >> 1)>{});
+    });
+  };
+
+  int it = blockIdx.x;
+  WoItem cur = item_of(it);
+  set_weights(cur);
+  load_step(0, qmm_const<0>{});
+  load_step(0, qmm_const<1>{});
+  int ring = 0;
+  for (;;) {
+    qmm_static_for<MT>([&](auto mc) {
+      constexpr int mt = mc;
+      xs[mt] = f32x4{0, 0, 0, 0};
+      qmm_static_for<NG>([&](auto gc) { acc[(int)gc][mt] = f32x4{0, 0, 0, 0}; });
+    });
+    int s = 0;
+    for (int c = 0; c < cur.n_chunks; ++c, ++ring) {
+      qmm_bare_barrier();  // chunk `ring` is there (the copying waves waited for it)
+      const int tile0 = (ring & 1) * CS - c * CS;
+      int s_end = min(cur.steps, (c + 1) * CS);
+      if (c + 1 == cur.n_chunks) --s_end;  // the item's last step fetches nothing more: it runs after the loop
+      for (; s < s_end; ++s) compute(tile0 + s, s + 1, qmm_const<1>{});
+      if (c + 1 == cur.n_chunks) compute(tile0 + s, 0, qmm_const<0>{});
+    }
+
+    // the next item's first weights are requested before this item's results are stored: a wait
+    // for them then does not include the stores
+    const WoItem done = cur;
+    const int it_next = it + (int)gridDim.x;
+    const bool more = it_next < n_items;
+    if (more) {
+      it = it_next;
+      cur = item_of(it);
+      set_weights(cur);
+      load_step(0, qmm_const<0>{});
+      load_step(0, qmm_const<1>{});
+    }
+
+    // ---- results: four consecutive channels of one row per lane ----
+    const int m0 = done.m0, n0 = done.n0;
+    if (a.split == 1) {
+      const WoDts<XT, UNI> dts(a);
+      // scales (and zero points) of this lane's channels first, all at once: loads inside the
+      // loop over row tiles would be waited for one after the other
+      uint32_t sraw[NG][4], zraw[NG][4];
+      qmm_static_for<NG>([&](auto gc) {
+        constexpr int gi = gc;
+        const int n = min(n0 + (wave * NG + gi) * 16 + 4 * g, N - 1);
+        wo_load4_raw(a.scale, n, N, dts.scale_dt, sraw[gi]);
+        if constexpr (HASZP) wo_load4_raw(a.zp, n, N, dts.zp_dt, zraw[gi]);
+      });
+      // the two store forms as two straight-line copies of the whole epilogue, chosen once
+      auto emit = [&](auto vecc) __attribute__((always_inline)) {
+        constexpr bool kVec = vecc != 0;
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          const int m = m0 + 16 * mt + r;
+          qmm_static_for<NG>([&](auto gc) {
+            constexpr int gi = gc;
+            const int n = n0 + (wave * NG + gi) * 16 + 4 * g;
+            if (m < M && n < N) {
+              if constexpr (kVec && UNI && !HASZP && XT == XLA_AMD_DT_BF16) {
+                wo_finish_store_bf16(a.out, m, n, N, sraw[gi], acc[gi][mt]);
+              } else {
+                float o[4];
+                wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, XT, o);
+                wo_store4<kVec>(a.out, m, n, N, o, dts.store_dt);
+              }
+            }
+          });
+        });
+      };
+      if ((N & 3) == 0) emit(qmm_const<1>{});
+      else emit(qmm_const<0>{});
+    } else {
+      const bool vec = (N & 3) == 0;
+      qmm_static_for<NG>([&](auto gc) {
+        constexpr int gi = gc;
+        const int n = n0 + (wave * NG + gi) * 16 + 4 * g;
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          const int m = m0 + 16 * mt + r;
+          if (m < M && n < N) {
+            float* p = a.part + ((size_t)done.ks * M + m) * N + n;
+            if (vec) *(f32x4*)p = acc[gi][mt];
+            else for (int v = 0; v < 4; ++v) if (n + v < N) p[v] = acc[gi][mt][v];
+          }
+        });
+      });
+      if constexpr (HASZP) {
+        // partial row sums of x: once per row tile and K slice (the first column tile's first wave, channel lanes 0..15)
+        if (n0 == 0 && wave == 0 && g == 0) {
+          qmm_static_for<MT>([&](auto mc) {
+            constexpr int mt = mc;
+            const int m = m0 + 16 * mt + r;
+            if (m < M) a.part_xs[(size_t)done.ks * M + m] = xs[mt][0];
+          });
+        }
+      }
+    }
+    if (!more) break;
+  }
+}
+
+// Compute units of the current device (asked once per device).
+int cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+template <int XT, int MT, int NG>
+int launch(const WoGemmArgs& a, hipStream_t stream) {
+  using Cfg = WoCfg<MT>;
+  const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + 64 * NG - 1) / (64 * NG)) * a.split;
+  const int steps = a.k_per_split / 128;
+  // one workgroup per compute unit (its LDS and registers leave room for no second one); each walks its share of the items
+  const int cus = cu_count();
+  const dim3 grid((unsigned)(items < cus ? items : cus)), block((kComputeWaves + kCopyWaves) * 64);
+  auto go = [&](auto kern) -> int {
+    static std::atomic<uint64_t> lds_set{0};
+    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20), lds_set, "weight_only_gemm hipFuncSetAttribute");
+    if (rc != XLA_AMD_QMM_OK) return rc;
+    // a workgroup with several items needs both chunk slots whatever the slice length
+    hipLaunchKernelGGL(kern, grid, block, Cfg::lds_bytes(items > cus ? (1 << 20) : steps), stream, a);
+    return QMM_CHECK_LAUNCH("weight_only_gemm launch");
+  };
+  // one dtype throughout (x, scale, zero point, dot, out, store): the epilogue's dtypes fold at compile time
+  const bool uni = a.scale_dt == XT && a.zp_dt == XT && a.dot_dt == XT && a.out_dt == XT && a.store_dt == XT;
+  if (uni) return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, true>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>);
+  return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, false>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, false>);
+}
+
+}  // namespace
+
+#define QMM_WO_CAT2(a, b, c) a##b##c
+#define QMM_WO_CAT(a, b, c) QMM_WO_CAT2(a, b, c)
+#if QMM_WO_XT == XLA_AMD_DT_BF16
+#define QMM_WO_UNIT_NAME QMM_WO_CAT(qmm_wo_launch_bf16_mt, QMM_WO_MT, )
+#else
+#define QMM_WO_UNIT_NAME QMM_WO_CAT(qmm_wo_launch_f16_mt, QMM_WO_MT, )
+#endif
+int QMM_WO_UNIT_NAME(const WoGemmArgs& a, int ng, hipStream_t stream) {
+  return ng == 4 ? launch<QMM_WO_XT, QMM_WO_MT, 4>(a, stream) : launch<QMM_WO_XT, QMM_WO_MT, 2>(a, stream);
+}
+
+#if QMM_WO_XT == XLA_AMD_DT_BF16 && QMM_WO_MT == 8
+namespace {
+
+// Adds the partial sums of a K split in slice order and finishes them: one thread per four
+// consecutive channels of one row.
+__global__ void __launch_bounds__(256) qmm_wo_gemm_finish_kernel(WoGemmArgs a, int x_dt) {
+  const int n4 = (a.N + 3) / 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)a.M * n4) return;
+  const int m = (int)(idx / n4), n = (int)(idx % n4) * 4;
+  const WoDts<0, false> dts(a);
+  uint32_t sraw[4], zraw[4] = {0, 0, 0, 0};
+  wo_load4_raw(a.scale, n, a.N, dts.scale_dt, sraw);
+  if (a.zp) wo_load4_raw(a.zp, n, a.N, dts.zp_dt, zraw);
+  f32x4 dot = {0, 0, 0, 0};
+  float xsum = 0.f;
+  for (int s = 0; s < a.split; ++s) {
+    const float* p = a.part + ((size_t)s * a.M + m) * a.N + n;
+    if ((a.N & 3) == 0) dot += *(const f32x4*)p;
+    else for (int v = 0; v < 4; ++v) if (n + v < a.N) dot[v] += p[v];
+    if (a.zp) xsum += a.part_xs[(size_t)s * a.M + m];
+  }
+  float o[4];
+  wo_finish4(dts, sraw, zraw, a.zp != nullptr, dot, xsum, x_dt, o);
+  if ((a.N & 3) == 0) wo_store4<true>(a.out, m, n, a.N, o, dts.store_dt);
+  else wo_store4<false>(a.out, m, n, a.N, o, dts.store_dt);
+}
+
+struct Plan {
+  int mt, ng, split, k_per_split;
+};
+
+// Tile and K split by shape.  Row tiles of 64 / 128 rows; 256 channels per workgroup
+// (128 when that is what fills the chip); K split over workgroups until about one workgroup
+// per compute unit is reached, in slices of at least 512 columns.
+// (with a zero point the 128-row tile keeps 128 channels per workgroup: the row sums of x take
+// the registers that the wider tile would need)
+Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
+  Plan p;
+  p.mt = M <= 64 ? 4 : 8;
+  const int64_t bm = 16 * p.mt;
+  const int64_t tiles_m = (M + bm - 1) / bm;
+  p.ng = 4;
+  if ((tiles_m * ((N + 255) / 256) < 192 && N > 128) || (has_zp && p.mt == 8)) p.ng = 2;
+  const int64_t tiles = tiles_m * ((N + 64 * p.ng - 1) / (64 * p.ng));
+  int64_t split = 1;
+  if (tiles < 192) split = (256 + tiles - 1) / tiles;
+  const int64_t blocks = K / 128;
+  int64_t per = (blocks + split - 1) / split;
+  if (per < 4) per = blocks < 4 ? blocks : 4;
+  split = (blocks + per - 1) / per;
+  p.split = (int)split;
+  p.k_per_split = (int)per * 128;
+  return p;
+}
+
+}  // namespace
+
+extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  size_t need = 0;
+  for (int zp = 0; zp < 2; ++zp) {  // the larger of the two plans: the size does not depend on the zero point
+    const Plan p = make_plan(M, N, K, zp != 0);
+    if (p.split > 1) {
+      const size_t b = ((size_t)p.split * (size_t)M * (size_t)N + (size_t)p.split * (size_t)M) * sizeof(float);
+      need = b > need ? b : need;
+    }
+  }
+  return need;
+}
+
+extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, const void* scale, const void* zp,
+                                            void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                                            int64_t K, int x_dt, int scale_dt, int zp_dt, int dot_dt, int out_dt,
+                                            int store_dt, void* stream) {
+  if (!x || !w_tiled || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: null pointer");
+  if (M < 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad sizes M=%lld N=%lld K=%lld",
+                                                 (long long)M, (long long)N, (long long)K);
+  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || !qmm_valid_dt(dot_dt) ||
+      !qmm_valid_dt(store_dt) || (zp && !qmm_valid_dt(zp_dt)))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad dtype enum");
+  if (out_dt != qmm_promote(x_dt, scale_dt))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: out dtype must be promote(x, scale)");
+  if (dot_dt != x_dt && dot_dt != XLA_AMD_DT_F32)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: dot dtype must be x's or f32");
+  if (x_dt == XLA_AMD_DT_F32) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x must be bf16 or f16");
+  if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: K=%lld must be a multiple of 128", (long long)K);
+  if (N > (1 << 30) || K > (1 << 24) || M > (1 << 24))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: dimension too large");
+  if (((uintptr_t)x | (uintptr_t)w_tiled) & 15)
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x and w must be 16-byte aligned");
+  if (((uintptr_t)out & 15) && (N & 3) == 0)
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: out must be 16-byte aligned");
+  if (M == 0) return XLA_AMD_QMM_OK;
+  const Plan p = make_plan(M, N, K, zp != nullptr);
+  WoGemmArgs a;
+  a.x = x; a.w = (const uint8_t*)w_tiled; a.scale = scale; a.zp = zp; a.out = out;
+  a.part = nullptr; a.part_xs = nullptr;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K;
+  a.k_per_split = p.k_per_split; a.split = p.split;
+  a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.dot_dt = dot_dt; a.out_dt = out_dt; a.store_dt = store_dt;
+  if (p.split > 1) {
+    const size_t need = ((size_t)p.split * (size_t)M * (size_t)N + (size_t)p.split * (size_t)M) * sizeof(float);
+    if (!workspace || workspace_bytes < need)
+      return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: workspace of %zu bytes, need %zu", workspace ? workspace_bytes : (size_t)0, need);
+    if ((uintptr_t)workspace & 15) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: workspace must be 16-byte aligned");
+    a.part = (float*)workspace;
+    a.part_xs = a.part + (size_t)p.split * (size_t)M * (size_t)N;
+  }
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (x_dt == XLA_AMD_DT_BF16) rc = p.mt == 4 ? qmm_wo_launch_bf16_mt4(a, p.ng, s) : qmm_wo_launch_bf16_mt8(a, p.ng, s);
+  else rc = p.mt == 4 ? qmm_wo_launch_f16_mt4(a, p.ng, s) : qmm_wo_launch_f16_mt8(a, p.ng, s);
+  if (rc != XLA_AMD_QMM_OK) return rc;
+  if (p.split > 1) {
+    const int64_t threads = M * ((N + 3) / 4);
+    hipLaunchKernelGGL(qmm_wo_gemm_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, a, x_dt);
+    rc = QMM_CHECK_LAUNCH("weight_only_gemm finish launch");
+  }
+  return rc;
+}
+#endif  // the unit with the entry points

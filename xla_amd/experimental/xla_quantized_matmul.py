@@ -35,7 +35,7 @@ def _overflow_policy() -> str:
 
 
 # Dispatch decisions, for tests and profiling (kernel id -> calls).
-counters = {"skinny_mfma": 0, "generic": 0, "w8a8_mfma": 0, "w8a8_generic": 0, "pack": 0, "pack_hit": 0}
+counters = {"skinny_mfma": 0, "wo_gemm": 0, "generic": 0, "w8a8_mfma": 0, "w8a8_generic": 0, "pack": 0, "pack_hit": 0}
 
 
 def _check_per_channel_quant_weight_dtype_shapes(input_dim, output_dim, w, w_scaler, zero_point):
@@ -219,7 +219,16 @@ def _weight_only_launch(x2, w, w_tiled, n, k, c, layout, bits, scaler, zero_poin
   zp_dt = _lib.dt(zero_point.dtype) if zero_point is not None else _lib.dt(x2.dtype)
   dts = (_lib.dt(x2.dtype), _lib.dt(scaler.dtype), zp_dt, _lib.dt(dot_dtype), _lib.dt(out_dtype),
          _lib.dt(store_dtype))
-  if kern == _lib.KERNEL_SKINNY_MFMA:
+  if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM:
+    wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
+    counters["wo_gemm"] += 1
+    nbytes = lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k)
+    workspace = torch.empty(nbytes, dtype=torch.uint8, device=x2.device) if nbytes else None
+    _lib.check(
+        lib.xla_amd_qmm_weight_only_gemm(x2.data_ptr(), wk.data_ptr(), scaler.data_ptr(), _lib.ptr(zero_point),
+                                         out.data_ptr(), _lib.ptr(workspace), nbytes, m, n, k, *dts, stream),
+        "weight_only_gemm")
+  elif kern == _lib.KERNEL_SKINNY_MFMA:
     wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
     counters["skinny_mfma"] += 1
     _lib.check(
