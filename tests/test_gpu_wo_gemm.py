@@ -52,7 +52,11 @@ def test_wo_gemm_shapes(ops, xdt, zp):
   # every row-tile height (32 / 64 / 128 rows), both tile widths, with and without a K split, M / N tails,
   # one to many K steps, several chunks of x
   for (m, n, k) in [(33, 256, 512), (64, 100, 1024), (17, 4096, 14336), (32, 1024, 4096), (128, 512, 128), (200, 333, 2560),
-                    (300, 700, 1024), (48, 64, 8192), (2, 16, 128), (130, 2048, 2048)]:
+                    (300, 700, 1024), (48, 64, 8192), (2, 16, 128), (130, 2048, 2048),
+                    # K slices of 3, 4 + 1, 4 + 3 and 4 + 4 + 3 steps (the two-deep weight ring's tails)
+                    (40, 96, 384), (64, 128, 640), (50, 200, 896), (64, 64, 1408),
+                    # more work items than compute units: workgroups walk several of them
+                    (60, 33024, 256)]:
     x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)
     z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(xdt) if zp else None
     exp = oracle.quantized_matmul(x, w, s, z)
