@@ -28,6 +28,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA (5.0 POP/s)
+BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA (2.5 PFLOP/s)
 
 N_OUT, K_IN = 14336, 4096
 TRAFFIC_BYTES_PER_LAUNCH = 60.4e6  # decode GEMV M=16, see profiles/skinny_gemv_cfg2_m16_hbm_traffic.md
@@ -164,7 +165,7 @@ def main():
           # elementwise kernel of known size); it is a profile result, not re-measured by this script
           "traffic": TRAFFIC_BYTES_PER_LAUNCH,
           "traffic_source": "profiles/skinny_gemv_cfg2_m16_hbm_traffic.md",
-          "kernel": "qmm_skinny_kernel<bf16, int8, MT=1>",
+          "kernel": "qmm_skinny_kernel<bf16, int8, MT=1> (4 computing + 4 copying waves)",
           "avg_launch_us": round(ev_ms * 1e3, 3),
       },
   }
@@ -221,7 +222,18 @@ def main():
         "tops_f32_out": round(ops4 / ev_g / 1e9, 1),
         "tops_end_to_end": round(ops4 / ev_e2e / 1e9, 1),
     }
-    del x4, xq, xsc
+    # weight-only prefill at the same shape (config 2's weight, M = 2048): the tiled bf16 GEMM with int8 weights
+    s2 = s_cpu.to(dev)
+    x4b = torch.randn(m4, K_IN, generator=cases.gen(2)).bfloat16().to(dev)  # config 2's activations: N(0, 1)
+    _, ev_wo, _ = time_calls([lambda: op(x4b, w0, s2)], steps4, 5, use_graph)
+    extra["weight_only_prefill_M2048"] = {
+        "us": round(ev_wo * 1e3, 2),
+        "roofline": {"bound": "mfma", "achieved": round(ops4 / ev_wo / 1e9, 1), "peak": BF16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(ops4 / ev_wo / 1e9 / BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "qmm_wo_gemm_kernel<bf16, 128 x 256 tile>"},
+        "vs_w8a8_end_to_end": round(ev_wo / ev_e2e, 2),
+    }
+    del x4, x4b, xq, xsc
 
     # Llama-3-8B decoder layer, 7 linears (config 5)
     shapes = {"q": (4096, 4096), "k": (1024, 4096), "v": (1024, 4096), "o": (4096, 4096),
@@ -231,11 +243,15 @@ def main():
     for name, (n, k) in shapes.items():
       w = torch.randint(-127, 128, (n, k), generator=g5, dtype=torch.int32).to(torch.int8).to(dev)
       layer[name] = (w, (torch.rand(n, generator=g5) * 0.01).to(dev))
+    # two more copies of the layer's weights: with three sets (654 MB) used in turn no weight is
+    # still in the 256 MB Infinity Cache when its turn comes again ("cold", what a model with many layers sees)
+    layer_sets = [layer] + [{k_: (v[0].clone(), v[1]) for k_, v in layer.items()} for _ in range(2)]
     for tag, m, qa in (("decode_M32", 32, False), ("prefill_M512", 512, True)):
       x_in = {4096: torch.randn(m, 4096, generator=g5).bfloat16().to(dev),
               14336: torch.randn(m, 14336, generator=g5).bfloat16().to(dev)}
 
       layer_s = {k_: (v[0], v[1] if qa else v[1].bfloat16()) for k_, v in layer.items()}
+      sets_s = [{k_: (v[0], v[1] if qa else v[1].bfloat16()) for k_, v in ls.items()} for ls in layer_sets]
 
       def run_layer():
         for name, (w, s) in layer_s.items():
@@ -243,7 +259,15 @@ def main():
 
       _, ev, _ = time_calls([run_layer], 20, 5, use_graph)
       extra[f"llama3_8b_layer_linears_{tag}"] = {"us": round(ev * 1e3, 2),
-                                                 "note": "weights (218 MB) stay cache-warm between iterations"}
+                                                 "note": "us: one set of weights (218 MB), cache-warm between iterations; "
+                                                         "us_cold: three sets in turn"}
+
+      def run_set(ls):
+        for name, (w, s) in ls.items():
+          op(x_in[w.shape[1]], w, s, quantize_activation=qa)
+
+      _, ev, _ = time_calls([(lambda ls=ls: run_set(ls)) for ls in sets_s], 21, 6, use_graph)
+      extra[f"llama3_8b_layer_linears_{tag}"]["us_cold"] = round(ev * 1e3, 2)
 
       # the same layer with q/k/v and gate/up concatenated along N: 4 launches instead of 7
       def cat(names):
@@ -259,7 +283,8 @@ def main():
 
       _, ev, _ = time_calls([run_fused], 20, 5, use_graph)
       extra[f"llama3_8b_layer_linears_{tag}"]["us_qkv_and_gate_up_fused"] = round(ev * 1e3, 2)
-      del fused_s
+      del fused_s, sets_s
+    del layer_sets[1:]
     # W8A8 GEMM with few output tiles: the down projection (4096 x 14336) at decode-sized M
     wd, sd = layer["down"]
     small = {}
@@ -305,6 +330,31 @@ def main():
       oracle.quantized_matmul(x16, w_cpu, s_cpu)
       t_runs.append(time.perf_counter() - t0)
     t_med = sorted(t_runs)[len(t_runs) // 2]
+    # the other configurations' CPU figures (bounded samples), next to their GPU entries
+    if extra:
+      def cpu_time(fn, budget_s=4.0, max_runs=20):
+        fn()
+        runs, t_begin = [], time.perf_counter()
+        while len(runs) < 3 or (time.perf_counter() - t_begin < budget_s and len(runs) < max_runs):
+          t0 = time.perf_counter()
+          fn()
+          runs.append(time.perf_counter() - t0)
+        return sorted(runs)[len(runs) // 2], len(runs)
+      x3, w3, s3, z3, _ = cases.blockwise(16, 4096, 4096, 128, 4, torch.bfloat16, symmetric=False, seed=4)
+      t3, n3 = cpu_time(lambda: oracle.quantized_matmul(x3, w3, s3, z3, block_size=128, int4_weight=True))
+      if "blockwise_int4_M16" in extra:
+        extra["blockwise_int4_M16"]["cpu_baseline"] = {
+            "value": round(extra["blockwise_int4_M16"]["algorithmic_bytes"] / t3 / 1e9, 3), "unit": "GB/s", "cores": cores,
+            "kind": "port", "sample": f"median of {n3} full calls of the same workload through the CPU oracle; {t3 * 1e3:.1f} ms per call"}
+      rows4 = 128  # of the 2048 rows: the CPU's int32 matmul takes seconds for all of them
+      x4c = cases.outlier_activations(2048, K_IN, torch.bfloat16, seed=1234)[:rows4].contiguous()
+      s4c = s_cpu.float()
+      t4, n4 = cpu_time(lambda: oracle.quantized_matmul(x4c, w_cpu, s4c, quantize_activation=True), budget_s=8.0, max_runs=10)
+      if "w8a8_prefill_M2048" in extra:
+        extra["w8a8_prefill_M2048"]["cpu_baseline"] = {
+            "value": round(2.0 * rows4 * N_OUT * K_IN / t4 / 1e12, 4), "unit": "TOP/s", "cores": cores, "kind": "port",
+            "sample": f"median of {n4} calls on the first {rows4} of the 2048 rows (quantize + int32 matmul + scales) "
+                      f"through the CPU oracle; {t4 * 1e3:.0f} ms per call"}
     result["cpu_baseline"] = {
         "value": round(bytes16 / t_med / 1e9, 3),
         "unit": "GB/s",

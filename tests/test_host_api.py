@@ -310,3 +310,14 @@ def test_fuse_quantized_linears_cpu():
     outs = fused(x).split([l.output_dim for l in lins], dim=-1)
     for l, o in zip(lins, outs):
       assert torch.equal(l(x), o), kwargs
+
+
+def test_no_kernel_of_the_built_library_spills_registers():
+  """The build writes every kernel's resources; a scratch frame (register spills) is a silent slowdown of several times."""
+  import json
+  from xla_amd import build
+  if not os.path.exists(build.RESOURCES_PATH):
+    pytest.skip("library not built by xla_amd.build in this tree")
+  kernels = json.load(open(build.RESOURCES_PATH))
+  assert len(kernels) > 50
+  assert [k for k in kernels if k.get("scratch_bytes_per_lane", 0) > 0] == []

@@ -6,6 +6,8 @@ needed to build.
 """
 import concurrent.futures
 import os
+import json
+import re
 import subprocess
 import sys
 
@@ -56,6 +58,31 @@ def _run(cmd):
   return out
 
 
+# Every kernel of the library must keep its registers: a kernel that spills to scratch memory
+# runs several times slower without failing any test.  The compiler reports each kernel's
+# resources (-Rpass-analysis=kernel-resource-usage); the build reads the report, writes it to
+# RESOURCES_PATH and refuses a kernel with a scratch frame.
+RESOURCES_PATH = os.path.join(OBJ_DIR, "kernel_resources.json")
+_REMARK = re.compile(r"remark:\s+(Function Name|VGPRs|AGPRs|ScratchSize \[bytes/lane\]|Occupancy \[waves/SIMD\]|"
+                     r"LDS Size \[bytes/block\]): (\S+)")
+
+
+def _kernel_resources(report: str, unit: str):
+  kernels, cur = [], None
+  for line in report.splitlines():
+    m = _REMARK.search(line)
+    if not m:
+      continue
+    key, val = m.group(1), m.group(2)
+    if key == "Function Name":
+      cur = {"unit": unit, "kernel": val}
+      kernels.append(cur)
+    elif cur is not None:
+      cur[{"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes_per_lane",
+           "Occupancy [waves/SIMD]": "waves_per_simd", "LDS Size [bytes/block]": "static_lds_bytes"}[key]] = int(val)
+  return kernels
+
+
 def build(verbose: bool = False, jobs: int = 8) -> str:
   os.makedirs(OBJ_DIR, exist_ok=True)
   objs = []
@@ -63,13 +90,28 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
   def compile_one(item):
     src, extra, name = item
     obj = os.path.join(OBJ_DIR, name)
-    out = _run([HIPCC] + FLAGS + extra + ["-c", os.path.join(CSRC, src), "-o", obj])
-    if verbose and out.strip():
-      print(out)
-    return obj
+    out = _run([HIPCC] + FLAGS + ["-Rpass-analysis=kernel-resource-usage"] + extra +
+               ["-c", os.path.join(CSRC, src), "-o", obj])
+    kernels = _kernel_resources(out, name)
+    if verbose:
+      # (a remark is followed by the source line it points at and a caret line)
+      rest = "\n".join(l for l in out.splitlines() if "kernel-resource-usage" not in l and
+                       not re.match(r"^\s*\d*\s*\|", l) and l.strip() != "^")
+      if rest.strip():
+        print(rest)
+    return obj, kernels
 
   with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-    objs = list(ex.map(compile_one, SOURCES))
+    results = list(ex.map(compile_one, SOURCES))
+  objs = [r[0] for r in results]
+  kernels = [k for r in results for k in r[1]]
+  with open(RESOURCES_PATH, "w") as f:
+    json.dump(kernels, f, indent=1)
+  spilling = [k for k in kernels if k.get("scratch_bytes_per_lane", 0) > 0]
+  if spilling:
+    raise RuntimeError("kernels with a scratch frame (register spills):\n" +
+                       "\n".join("  %s: %s (%d bytes per lane, %d VGPRs)" % (k["unit"], k["kernel"], k["scratch_bytes_per_lane"],
+                                                                            k.get("vgprs", -1)) for k in spilling))
   tmp = LIB_PATH + ".tmp"
   _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] + objs)
   os.replace(tmp, LIB_PATH)

@@ -107,13 +107,9 @@ template <int XT> __device__ __forceinline__ i32x4 ones_frag() {
 template <int MT> struct WoCfg {
   static constexpr int BM = 16 * MT;
   static constexpr int X_TILE = BM * 256;                      // bytes of the x columns of one step (128 columns, 2-byte x)
-  // Weight blocks in flight per wave and channel group (register ring): one step for the
-  // 128-row tile, whose accumulators leave no room for more and whose steps are long; two for
-  // the smaller tiles, whose short steps would otherwise wait for memory every time.
-  static constexpr int P = MT >= 8 ? 1 : 2;
-  static constexpr int kFit = kLds / (2 * X_TILE) / P * P;     // steps per chunk slot that fit twice (whole trips around the ring)
+  static constexpr int kFit = kLds / (2 * X_TILE);             // steps per chunk slot that fit twice
   static constexpr int CS = kFit < 8 ? kFit : 8;               // steps per chunk
-  static_assert(CS >= P, "two chunk slots must fit in LDS");
+  static_assert(CS >= 1, "two chunk slots must fit in LDS");
   static constexpr int lds_bytes(int steps) { return (steps <= CS ? steps : 2 * CS) * X_TILE; }
 };
 
@@ -266,9 +262,8 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   // wave w owns the channel groups (n0/16 + w*NG) .. + NG-1 of the item's column tile
   const int n_blk = K / 128;  // blocks per channel group in the tiled weight
   const int groups = (N + 15) / 16;
-  constexpr int P = Cfg::P;
   const uint8_t* wp[NG];
-  i32x4 wreg[P][NG][2];  // ring slot s % P holds the block of step s
+  i32x4 wreg[NG][2];
   auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
@@ -276,28 +271,18 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * 2048 + lane * 16;
     });
   };
-  auto load_half = [&](int blk, auto slotc, auto hc) __attribute__((always_inline)) {
-    constexpr int slot = slotc, h = hc;
+  auto load_step = [&](int blk, auto hc) __attribute__((always_inline)) {
+    constexpr int h = hc;
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      wreg[slot][gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * 2048 + h * 1024));
-    });
-  };
-  // the first P blocks of an item (a block past the end of a short item is the last one again: never used)
-  auto load_first = [&](const WoItem& w) __attribute__((always_inline)) {
-    qmm_static_for<P>([&](auto pc) {
-      constexpr int slot = pc;
-      const int blk = min(slot, w.steps - 1);
-      load_half(blk, qmm_const<slot>{}, qmm_const<0>{});
-      load_half(blk, qmm_const<slot>{}, qmm_const<1>{});
+      wreg[gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * 2048 + h * 1024));
     });
   };
 
   f32x4 acc[NG][MT], xs[MT];
-  // one step (128 columns) out of LDS tile `tile` with the weights of ring slot SLOT; with
-  // REFILL the slot's registers are refilled with block `next` as soon as each half has been used
-  auto compute = [&](int tile, int next, auto slotc, auto refillc) __attribute__((always_inline)) {
-    constexpr int slot = slotc;
+  // one step (128 columns) out of LDS tile `tile`; the weight registers are refilled with
+  // block `next` as soon as each half has been used
+  auto compute = [&](int tile, int next, auto refillc) __attribute__((always_inline)) {
     constexpr bool kRefill = refillc != 0;
     const char* xbase = smem + tile * X_TILE;
     qmm_static_for<4>([&](auto jc) {
@@ -309,7 +294,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       });
       qmm_static_for<NG>([&](auto gc) {
         constexpr int gi = gc;
-        const i32x4 src = wreg[slot][gi][j >> 1];
+        const i32x4 src = wreg[gi][j >> 1];
         const i32x4 af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
         qmm_static_for<MT>([&](auto mc) {
           constexpr int mt = mc;
@@ -322,23 +307,15 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
           xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt], xs[mt]);
         });
       }
-      if constexpr (kRefill && (j & 1)) load_half(next, qmm_const<slot>{}, qmm_const<(j >> 1)>{});
-    });
-  };
-  // P consecutive steps starting at step s (s % P == 0) of which `live` exist; NREF of them refill
-  // their slot (the refills are compile-time so that the loads in flight stay countable)
-  auto compute_group = [&](int tile, int s, int live, auto nrefc) __attribute__((always_inline)) {
-    constexpr int nref = nrefc;
-    qmm_static_for<P>([&](auto pc) {
-      constexpr int slot = pc;
-      if (slot == 0 || slot < live) compute(tile + slot, s + slot + P, qmm_const<slot>{}, qmm_const<(slot < nref ? 1 : 0)>{});
+      if constexpr (kRefill && (j & 1)) load_step(next, qmm_const<(j >> 1)>{});
     });
   };
 
   int it = blockIdx.x;
   WoItem cur = item_of(it);
   set_weights(cur);
-  load_first(cur);
+  load_step(0, qmm_const<0>{});
+  load_step(0, qmm_const<1>{});
   int ring = 0;
   for (;;) {
     qmm_static_for<MT>([&](auto mc) {
@@ -350,19 +327,10 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     for (int c = 0; c < cur.n_chunks; ++c, ++ring) {
       qmm_bare_barrier();  // chunk `ring` is there (the copying waves waited for it)
       const int tile0 = (ring & 1) * CS - c * CS;
-      const int s_end = min(cur.steps, (c + 1) * CS);
-      // groups of P steps (a chunk holds whole groups); the item's last P steps fetch nothing more
-      for (; s < s_end; s += P) {
-        const int left = cur.steps - s;
-        if (left >= 2 * P) {
-          compute_group(tile0 + s, s, P, qmm_const<P>{});
-        } else if constexpr (P == 2) {
-          if (left == 3) compute_group(tile0 + s, s, 2, qmm_const<1>{});
-          else compute_group(tile0 + s, s, left, qmm_const<0>{});
-        } else {
-          compute_group(tile0 + s, s, 1, qmm_const<0>{});
-        }
-      }
+      int s_end = min(cur.steps, (c + 1) * CS);
+      if (c + 1 == cur.n_chunks) --s_end;  // the item's last step fetches nothing more: it runs after the loop
+      for (; s < s_end; ++s) compute(tile0 + s, s + 1, qmm_const<1>{});
+      if (c + 1 == cur.n_chunks) compute(tile0 + s, 0, qmm_const<0>{});
     }
 
     // the next item's first weights are requested before this item's results are stored: a wait
@@ -374,7 +342,8 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       it = it_next;
       cur = item_of(it);
       set_weights(cur);
-      load_first(cur);
+      load_step(0, qmm_const<0>{});
+      load_step(0, qmm_const<1>{});
     }
 
     // ---- results: four consecutive channels of one row per lane ----
@@ -474,8 +443,14 @@ int launch(const WoGemmArgs& a, hipStream_t stream) {
   };
   // one dtype throughout (x, scale, zero point, dot, out, store): the epilogue's dtypes fold at compile time
   const bool uni = a.scale_dt == XT && a.zp_dt == XT && a.dot_dt == XT && a.out_dt == XT && a.store_dt == XT;
-  if (uni) return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, true>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>);
-  return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, false>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, false>);
+  if constexpr (MT == 8 && NG == 4) {
+    // (the 128 x 256 tile with the row sums of x does not fit the register file: the plan never asks for it)
+    if (a.zp) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: no 128 x 256 tile with a zero point");
+    return uni ? go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, false>);
+  } else {
+    if (uni) return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, true>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>);
+    return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, false>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, false>);
+  }
 }
 
 }  // namespace
