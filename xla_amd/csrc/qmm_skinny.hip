@@ -42,21 +42,7 @@
 #error "compile with -DQMM_SKINNY_XT=<XLA_AMD_DT_* value>"
 #endif
 
-struct SkinnyArgs {
-  const void* x;
-  const uint8_t* w;  // K-major packed weight
-  const void* scale;
-  const void* zp;
-  void* out;
-  int M, N, K, C;  // M = rows of this pass (<= 16*MT)
-  int scale_dt, zp_dt, out_dt;
-  int dot_dt;    // dtype the dot product is rounded to before it is scaled (per-channel only)
-  int store_dt;  // dtype of the stored tensor (out_dt, or a final cast of it)
-};
-
-int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
-int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
-int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
+#include "qmm_skinny.h"
 
 namespace {
 
@@ -206,7 +192,11 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rw = wave % RW, kw = wave / RW;
   const int r = lane & 15, g = lane >> 4;
-  const int K = a.K, N = a.N, M = a.M, C = a.C;
+  // this workgroup's K slice: columns k_begin .. k_begin + K of rows that hold ldk columns
+  const int ldk = a.K;
+  const int k_begin = (int)blockIdx.y * a.k_per_slice;
+  const int K = min(a.k_per_slice, ldk - k_begin);
+  const int N = a.N, M = a.M, C = a.slices > 1 ? K : a.C;
   const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
   const int x_dt = XT;
   const int scale_dt = UNI ? XT : a.scale_dt, zp_dt = UNI ? XT : a.zp_dt, out_dt = UNI ? XT : a.out_dt;
@@ -218,11 +208,11 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // 128 columns, one block of BLK bytes; the blocks of a group follow each other
   // along K, so a wave streams one contiguous region.  Lane l of a 1 KB load
   // takes bytes [16 l, 16 l + 16): its own operand fragment.
-  const int n_blk = K / 128;                                    // blocks per channel group
+  const int n_blk = K / 128;                                    // blocks of this slice per channel group
   const int groups = (N + 15) / 16;
   const int my_group = min((int)blockIdx.x * RW + rw, groups - 1);  // tail groups re-read the last one
-  const uint8_t* const w_base = a.w + (size_t)my_group * n_blk * BLK + lane * 16;
-  const char* const x_base = (const char*)a.x;
+  const uint8_t* const w_base = a.w + ((size_t)my_group * (ldk / 128) + k_begin / 128) * BLK + lane * 16;
+  const char* const x_base = (const char*)a.x + (size_t)k_begin * XB;
   // x: copied global -> LDS without passing registers (global_load_lds_dwordx4:
   // lane l of an instruction lands at base + 16 l), 1 KB of one row per
   // instruction.  The XOR swizzle of the tile is applied on the source side: LDS
@@ -270,7 +260,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const int nst = min(CS, steps_total - c0);
     char* const slot = smem + (kSlots == 2 ? (c & 1) * (CS * X_TILE) : 0);
     for (int row = copy_wave; row < x_rows; row += kCopyWaves) {
-      const char* xrow = x_base + (size_t)row * ((size_t)K * XB) + (size_t)c0 * XROW;  // row `row`, first column of the chunk
+      const char* xrow = x_base + (size_t)row * ((size_t)ldk * XB) + (size_t)c0 * XROW;  // row `row`, first column of the chunk
       char* lrow = slot + row * XROW;
       const int sw = row & 15;
       for (int t = 0; t < nst; ++t) {
@@ -664,7 +654,28 @@ qmm_skinny_kernel(SkinnyArgs a) {
       }
     });
   }
-  if constexpr (RED == kRedRaw) block_epilogue(0, qmm_const<0>{});  // the single block ends here
+  if constexpr (RED == kRedRaw) {
+    if (a.slices > 1) {
+      // one K slice of several: the raw sums go to the workspace, a second kernel adds the slices and finishes them
+      const int slice = blockIdx.y;
+      qmm_static_for<MT>([&](auto mc) {
+        constexpr int mt = mc;
+        const int m = 16 * mt + r;
+        const int n = n_wave + 4 * g;
+        if (m < M && n < N) {
+          float* p = a.part + ((size_t)slice * M + m) * N + n;
+          const f32x4 t = {acc[mt][0] + accb[mt][0], acc[mt][1] + accb[mt][1], acc[mt][2] + accb[mt][2], acc[mt][3] + accb[mt][3]};
+          if ((N & 3) == 0) *(f32x4*)p = t;
+          else for (int v = 0; v < 4; ++v) if (n + v < N) p[v] = t[v];
+          if constexpr (NEEDXS) {
+            if (n_wave == 0 && g == 0) a.part_xs[(size_t)slice * M + m] = xs[mt][0];
+          }
+        }
+      });
+      return;
+    }
+    block_epilogue(0, qmm_const<0>{});  // the single block ends here
+  }
 
   qmm_static_for<MT>([&](auto mc) {
     constexpr int mt = mc;
@@ -715,8 +726,9 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
     const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20, kSlots), lds_set, "weight_only_skinny hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
-    const int steps = (a.K + Cfg::KS - 1) / Cfg::KS;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3((NW + skinny_copier_waves<MT, RED>()) * 64), Cfg::lds_bytes(steps, kSlots), stream, a);
+    const int steps = (a.k_per_slice + Cfg::KS - 1) / Cfg::KS;
+    hipLaunchKernelGGL(kern, dim3(blocks, (unsigned)a.slices), dim3((NW + skinny_copier_waves<MT, RED>()) * 64),
+                       Cfg::lds_bytes(steps, kSlots), stream, a);
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
@@ -744,11 +756,12 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
   constexpr int KS = BITS == 8 ? kWSeg : 2 * kWSeg;
   const bool perch = a.C == a.K;
   const bool can_split = perch || (KS % a.C == 0);
-  const int steps = (a.K + KS - 1) / KS;
+  const int steps = (a.k_per_slice + KS - 1) / KS;  // of one workgroup
+  const int64_t spread = (int64_t)a.N * a.slices;   // K slices over workgroups multiply the workgroups like channels do
   int kw = 1;
   if (can_split) {
-    if (a.N < 200 * 64 && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
-    if (a.N < 200 * 32 && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
+    if (spread < 200 * 64 && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
+    if (spread < 200 * 32 && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
   }
   if (kw == 1) {
     return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
@@ -832,6 +845,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
     a.N = (int)N; a.K = (int)K; a.C = (int)C;
     a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.out_dt = out_dt;
     a.dot_dt = dot_dt; a.store_dt = store_dt;
+    a.k_per_slice = (int)K; a.slices = 1; a.part = nullptr; a.part_xs = nullptr;
     int rc;
     if (x_dt == XLA_AMD_DT_BF16) rc = qmm_skinny_launch_bf16(a, bits, zp != nullptr, (hipStream_t)stream);
     else if (x_dt == XLA_AMD_DT_F16) rc = qmm_skinny_launch_f16(a, bits, zp != nullptr, (hipStream_t)stream);

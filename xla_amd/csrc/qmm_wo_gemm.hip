@@ -33,6 +33,7 @@
 // -DQMM_WO_MT=4|8) so that the units build in parallel; the unit of bf16 with MT = 8 also
 // holds the second kernel of a K split and the C entry points.
 #include "qmm_common.h"
+#include "qmm_skinny.h"
 
 #if !defined(QMM_WO_XT) || !defined(QMM_WO_MT)
 #error "compile with -DQMM_WO_XT=<XLA_AMD_DT_BF16|XLA_AMD_DT_F16 value> -DQMM_WO_MT=<4|8>"
@@ -526,6 +527,11 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
 
 extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  if (M <= 32) {  // the weight-streaming kernel over K slices
+    int per;
+    const int slices = qmm_skinny_k_slices(M, N, K, &per);
+    if (slices > 1) return ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
+  }
   size_t need = 0;
   for (int zp = 0; zp < 2; ++zp) {  // the larger of the two plans: the size does not depend on the zero point
     const Plan p = make_plan(M, N, K, zp != 0);
@@ -560,6 +566,33 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
   if (((uintptr_t)out & 15) && (N & 3) == 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: out must be 16-byte aligned");
   if (M == 0) return XLA_AMD_QMM_OK;
+  if (M <= 32) {
+    // few rows: the weight-streaming kernel over K slices, when that is what its plan says and the workspace is there
+    int per;
+    const int slices = qmm_skinny_k_slices(M, N, K, &per);
+    const size_t need = ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
+    if (slices > 1 && workspace && workspace_bytes >= need && (((uintptr_t)workspace) & 15) == 0) {
+      SkinnyArgs k;
+      k.x = x; k.w = (const uint8_t*)w_tiled; k.scale = scale; k.zp = zp; k.out = out;
+      k.M = (int)M; k.N = (int)N; k.K = (int)K; k.C = (int)K;
+      k.scale_dt = scale_dt; k.zp_dt = zp ? zp_dt : x_dt; k.out_dt = out_dt; k.dot_dt = dot_dt; k.store_dt = store_dt;
+      k.k_per_slice = per; k.slices = slices;
+      k.part = (float*)workspace;
+      k.part_xs = k.part + (size_t)slices * (size_t)M * (size_t)N;
+      int rc = x_dt == XLA_AMD_DT_BF16 ? qmm_skinny_launch_bf16(k, 8, zp != nullptr, (hipStream_t)stream)
+                                       : qmm_skinny_launch_f16(k, 8, zp != nullptr, (hipStream_t)stream);
+      if (rc != XLA_AMD_QMM_OK) return rc;
+      WoGemmArgs f;
+      f.x = x; f.w = (const uint8_t*)w_tiled; f.scale = scale; f.zp = zp; f.out = out;
+      f.part = k.part; f.part_xs = k.part_xs;
+      f.M = (int)M; f.N = (int)N; f.K = (int)K; f.k_per_split = per; f.split = slices;
+      f.scale_dt = scale_dt; f.zp_dt = zp ? zp_dt : x_dt; f.dot_dt = dot_dt; f.out_dt = out_dt; f.store_dt = store_dt;
+      const int64_t threads = M * ((N + 3) / 4);
+      hipLaunchKernelGGL(qmm_wo_gemm_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                         (hipStream_t)stream, f, x_dt);
+      return QMM_CHECK_LAUNCH("weight_only_gemm finish launch");
+    }
+  }
   const Plan p = make_plan(M, N, K, zp != nullptr);
   WoGemmArgs a;
   a.x = x; a.w = (const uint8_t*)w_tiled; a.scale = scale; a.zp = zp; a.out = out;
