@@ -483,12 +483,24 @@ __global__ void __launch_bounds__(256) qmm_wo_gemm_finish_kernel(WoGemmArgs a, i
   if (a.zp) wo_load4_raw(a.zp, n, a.N, dts.zp_dt, zraw);
   f32x4 dot = {0, 0, 0, 0};
   float xsum = 0.f;
-  for (int s = 0; s < a.split; ++s) {
-    const float* p = a.part + ((size_t)s * a.M + m) * a.N + n;
-    if ((a.N & 3) == 0) dot += *(const f32x4*)p;
-    else for (int v = 0; v < 4; ++v) if (n + v < a.N) dot[v] += p[v];
-    if (a.zp) xsum += a.part_xs[(size_t)s * a.M + m];
+  const size_t slice = (size_t)a.M * a.N;
+  const float* p = a.part + (size_t)m * a.N + n;
+  int s = 0;
+  if ((a.N & 3) == 0) {
+    // four slices' loads in flight at a time (the slices come from memory: one load after the
+    // other would cost a memory latency each); the additions stay in slice order
+    for (; s + 4 <= a.split; s += 4) {
+      const f32x4 p0 = *(const f32x4*)(p + (size_t)s * slice), p1 = *(const f32x4*)(p + (size_t)(s + 1) * slice);
+      const f32x4 p2 = *(const f32x4*)(p + (size_t)(s + 2) * slice), p3 = *(const f32x4*)(p + (size_t)(s + 3) * slice);
+      dot += p0; dot += p1; dot += p2; dot += p3;
+    }
+    for (; s < a.split; ++s) dot += *(const f32x4*)(p + (size_t)s * slice);
+  } else {
+    for (; s < a.split; ++s)
+      for (int v = 0; v < 4; ++v) if (n + v < a.N) dot[v] += p[(size_t)s * slice + v];
   }
+  if (a.zp)
+    for (int t = 0; t < a.split; ++t) xsum += a.part_xs[(size_t)t * a.M + m];
   float o[4];
   wo_finish4(dts, sraw, zraw, a.zp != nullptr, dot, xsum, x_dt, o);
   if ((a.N & 3) == 0) wo_store4<true>(a.out, m, n, a.N, o, dts.store_dt);
