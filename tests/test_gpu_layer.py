@@ -107,7 +107,13 @@ def test_config5_fused_projections(ops, layer):
       fused = fuse_quantized_linears(mods)
       outs = fused(x).split([l.output_dim for l in mods], dim=-1)
       for nm, l, o in zip(names, mods, outs):
-        assert torch.equal(l(x), o), (qa, nm)
+        if qa:  # int32 sums: exact in any order
+          assert torch.equal(l(x), o), (qa, nm)
+        else:
+          # float sums: the number of output channels decides how K is split over the waves of a
+          # workgroup, so the wide launch may add in another order: a last-place flip here and there
+          sep = l(x)
+          assert (sep != o).float().mean().item() < 0.02 and cases.rel_l2(o.cpu(), sep.cpu()) < 1e-3, (qa, nm)
       w0, s0 = layer[names[0]]
       exp = oracle.quantized_matmul(x.cpu()[:8], w0, s0 if qa else s0.bfloat16(), quantize_activation=qa)
       check(outs[0][:8], exp, f"fused {names} qa={qa}")

@@ -748,20 +748,25 @@ int launch_zp(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
   }
 }
 
-// k-splits per workgroup: as few as keep >= ~200 workgroups, and only where the
-// reduction is defined (per-channel, or whole quantization blocks per step) and
-// the wider x tile still fits in LDS.
+// K split over the waves of a workgroup (KW = 1, 2, 4: 64, 32, 16 channels per workgroup): the
+// largest that still gives one workgroup per compute unit at most (256 of them), where the
+// reduction is defined (per-channel, or whole quantization blocks per step) and the wider x tile
+// fits in LDS.  More workgroups than compute units is a second, partly empty round and more
+// copies of x: measured at M = 32, K = 4096 with cold weights, N = 6144 takes 16.9 us in 384
+// workgroups of 16 channels and 11.5 us in 192 of 32; N = 11008 takes 21.1 us in 344 workgroups of
+// 32 channels and 13.4 us in 172 of 64.
 template <int XT, int BITS, int MT>
 int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
   constexpr int KS = BITS == 8 ? kWSeg : 2 * kWSeg;
+  constexpr int64_t kComputeUnits = 256;
   const bool perch = a.C == a.K;
   const bool can_split = perch || (KS % a.C == 0);
   const int steps = (a.k_per_slice + KS - 1) / KS;  // of one workgroup
-  const int64_t spread = (int64_t)a.N * a.slices;   // K slices over workgroups multiply the workgroups like channels do
+  auto workgroups = [&](int kw_) { return ((int64_t)a.N + 64 / kw_ - 1) / (64 / kw_) * a.slices; };  // K slices multiply them too
   int kw = 1;
   if (can_split) {
-    if (spread < 200 * 64 && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
-    if (spread < 200 * 32 && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
+    if (workgroups(2) <= kComputeUnits && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
+    if (workgroups(4) <= kComputeUnits && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
   }
   if (kw == 1) {
     return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
