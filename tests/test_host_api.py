@@ -52,6 +52,19 @@ def test_dispatcher_regimes():
   assert d(1, 4096, 4096, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA
   assert d(3, 8, 5, 5, 8, _lib.DT_F32, 0) == _lib.KERNEL_GENERIC
   assert d(3, 8, 6, 2, 8, _lib.DT_F32, 0) == _lib.KERNEL_GENERIC
+  # weight-only, per-channel int8, 2-byte x: more than 32 rows take the tiled GEMM; so do few rows against few
+  # channels and a long K (the streaming kernel over K slices, behind the same entry point with a workspace)
+  assert d(33, 14336, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
+  assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
+  assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F32, 0) == _lib.KERNEL_SKINNY_MFMA
+  assert d(2048, 4096, 4096, 128, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # blockwise
+  assert d(2048, 14336, 4096, 4096, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA    # int4
+  assert d(32, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
+  assert d(4, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # too few rows of x to matter
+  assert d(32, 4096, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA       # K too short for slices
+  assert d(32, 14336, 8192, 8192, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # enough workgroups already
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336) == 4 * (32 * 4096 + 32) * 4  # four K slices
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 14336, 4096) == 0
   assert d(2048, 14336, 4096, 4096, 8, _lib.DT_BF16, 1) == _lib.KERNEL_W8A8_MFMA
   assert d(3, 8, 5, 5, 8, _lib.DT_F32, 1) == _lib.KERNEL_W8A8_GENERIC
   tile = (ctypes.c_int32 * 3)()
