@@ -136,7 +136,8 @@ def test_int4_per_channel(ops):
 @pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("policy", ["saturate", "wrap"])
 def test_quantize_per_token_bit_exact(ops, xdt, policy):
-  for (m, k) in [(64, 4096), (5, 37), (3, 8), (1, 16384)]:
+  # rows kept in registers (2, 4, 8 vector steps per thread), one-element steps, and a row read twice (K > 16384)
+  for (m, k) in [(64, 4096), (5, 37), (3, 8), (1, 16384), (4, 8192), (3, 14336), (2, 20480)]:
     x = cases.outlier_activations(m, k, xdt, seed=11 + m)
     if m >= 3:
       x[1] = 0  # all-zero row

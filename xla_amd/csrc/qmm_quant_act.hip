@@ -1,5 +1,5 @@
 // Per-token dynamic int8 quantization of activations (HBM-bound elementwise +
-// row reduction).  One workgroup per row.  Rows of up to 8192 elements stay in
+// row reduction).  One workgroup per row.  Rows of up to 16384 elements stay in
 // registers between the abs-max pass and the quantize pass (x is read exactly
 // once); longer rows are read a second time, which hits L2.
 //
@@ -168,6 +168,8 @@ int launch(const void* x, int8_t* xq, void* x_scale, int32_t* x_sum, int64_t M, 
     hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 2>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
   else if (K <= 4 * kThreads * 8)
     hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 4>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
+  else if (K <= 8 * kThreads * 8)
+    hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 8>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
   else
     hipLaunchKernelGGL((qmm_quantize_kernel<XT, 8, 0>), grid, block, 0, stream, x, xq, x_scale, x_sum, K, scale_out_dt, policy);
   return QMM_CHECK_LAUNCH("quantize_per_token launch");
