@@ -574,3 +574,19 @@ def test_fused_linears_on_gpu(ops):
     outs = fused(x).split([l.output_dim for l in lins], dim=-1)
     for l, o in zip(lins, outs):
       assert torch.equal(l(x), o), kwargs
+
+
+def test_w8a8_f16_scaler_overflow_like_the_reference(ops):
+  """With an f16 scaler the reference converts the int32 sums to f16 before it scales them: sums beyond 65504
+  become inf there, and here at the same places with the same sign."""
+  for (m, n, k, zp) in [(7, 512, 640, True), (31, 16, 256, False), (300, 333, 8704, True)]:
+    x = cases.outlier_activations(m, k, torch.float16, seed=5)
+    _, w, s, _ = cases.per_channel_int8(1, n, k, torch.float16, torch.float16, seed=5)
+    z = (torch.randn(n, generator=cases.gen(6)) * 0.01).half() if zp else None
+    exp = oracle.quantized_matmul(x, w, s, z, quantize_activation=True)
+    out = torch.ops.xla.quantized_matmul(x.cuda(), w.cuda(), s.cuda(), None if z is None else z.cuda(), -1, False, True).cpu()
+    fin = torch.isfinite(exp)
+    assert (~fin).any() and not exp.isnan().any()
+    assert torch.equal(torch.isfinite(out), fin) and torch.equal(out[~fin], exp[~fin]), (m, n, k)
+    zero = torch.zeros_like(out)
+    assert cases.within_tolerance(torch.where(fin, out, zero), torch.where(fin, exp, zero)), (m, n, k)
