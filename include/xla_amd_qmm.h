@@ -173,7 +173,11 @@ size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_
  * Per-channel int8 weights only (w_tiled from xla_amd_qmm_tile_weight with
  * bits == 8), x [M,K] bf16 or f16, K % 128 == 0; other cases return
  * XLA_AMD_QMM_EUNSUPPORTED (the streaming kernel takes them).  dtype arguments
- * as for xla_amd_qmm_weight_only_skinny.  When K is split over workgroups the
+ * as for xla_amd_qmm_weight_only_skinny.  With at most 32 rows, few output
+ * channels and a long K (where xla_amd_qmm_dispatch returns this kernel for such
+ * an M) the call runs the streaming kernel over K slices instead, one slice of 64
+ * channels per workgroup, and a second kernel adds the slices in slice order.
+ * When K is split over workgroups the
  * partial sums live in `workspace` (device memory of at least
  * xla_amd_qmm_weight_only_gemm_workspace_bytes(M, N, K) bytes, 16-byte
  * aligned, free again when the call's work has completed); it may be NULL
