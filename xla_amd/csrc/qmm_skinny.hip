@@ -48,7 +48,7 @@ namespace {
 
 constexpr int kWaves = 4;         // waves per workgroup of the standard shape
 constexpr int kWSeg = 512;        // weight bytes per row per step of the standard shape
-constexpr int kLdsLimit = 160 * 1024;
+constexpr int kLdsLimit = 144 * 1024;  // of x in LDS; the 16 KB above it hold the blockwise scales of the resident chunks
 
 // ---- operand fragments --------------------------------------------------------
 __device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
@@ -172,6 +172,19 @@ template <typename Cfg, int MT, int RED, int KW> constexpr int skinny_slots() {
   return (skinny_copier_waves<MT, RED>() > 0 && Cfg::CS2 >= Cfg::P * KW) ? 2 : 1;
 }
 
+// Blockwise launches keep, next to every resident x tile, the scale and zero point of each of its
+// 128-column sub-steps (those of the quantization block the sub-step lies in) for the workgroup's
+// channels: "entries" of 16 * RW values, indexed like the x tiles.  The waves that copy a chunk of x
+// copy its entries too; the computing waves then read 4 channels' values with one LDS read instead of
+// fetching them from global memory between the weight loads.
+template <typename Cfg, int XT, int MT, int RED, int KW> constexpr int skinny_scale_bytes() {
+  if (RED == 1 /*kRedRaw*/) return 0;
+  constexpr int slots = skinny_slots<Cfg, MT, RED, KW>();
+  constexpr int cs = slots == 2 ? Cfg::CS2 : Cfg::CS1;
+  constexpr int entry = 16 * Cfg::RW * (XT == XLA_AMD_DT_F32 ? 4 : 2);
+  return 2 * slots * cs * Cfg::SUB * entry;  // scale and zero point
+}
+
 // UNI: scale, zero point, dot product, result and stored tensor all have x's dtype (the common
 // case, and the only one for blockwise weights): the dtypes are compile-time constants then, and
 // the code that runs once per wave (epilogue, scale conversion) has no dtype branches.
@@ -255,10 +268,41 @@ qmm_skinny_kernel(SkinnyArgs a) {
   constexpr int kCopyWaves = kCopiers > 0 ? kCopiers : NW;
   const int copy_wave = kCopiers > 0 ? wave - NW : wave;
   const int n_chunks = (steps_total + CS - 1) / CS;
+  // LDS: [blockwise scale entries][x tiles]
+  constexpr int kSclBytes = skinny_scale_bytes<Cfg, XT, MT, RED, KW>();
+  static_assert(kSclBytes <= 16 * 1024, "scale entries must fit above the x tiles");
+  constexpr int SE = XT == XLA_AMD_DT_F32 ? 4 : 2;   // bytes of a blockwise scale (x's dtype)
+  constexpr int kEntryBytes = 16 * RW * SE;          // one entry: the workgroup's channels
+  constexpr int kSclTensor = kSclBytes / 2;          // the scales' entries, then the zero points'
+  char* const xsm = smem + kSclBytes;
+  const int n_sblk = K / C;
+  const int c_shift = (C & (C - 1)) == 0 ? __builtin_ctz(C) : -1;  // block size a power of two: shift instead of divide
   auto x_chunk_load = [&](int c) __attribute__((always_inline)) {
     const int c0 = c * CS;
     const int nst = min(CS, steps_total - c0);
-    char* const slot = smem + (kSlots == 2 ? (c & 1) * (CS * X_TILE) : 0);
+    if constexpr (RED != kRedRaw) {
+      // entries of this chunk's tiles, 4 bytes per lane and instruction (256 bytes of consecutive entries):
+      // entry e of the slot is sub-step e of the chunk, columns (c0 * SUB + e) * 128 ...
+      constexpr int kPieces = kEntryBytes / 4;   // 4-byte pieces per entry (<= 64)
+      constexpr int kEpi = 64 / kPieces;         // entries per instruction
+      static_assert(kPieces <= 64 && (CS * SUB) % kEpi == 0, "whole instructions per chunk");
+      constexpr int kInstr = CS * SUB / kEpi;
+      const int n_wg0 = n_wave - 16 * rw;        // the workgroup's first channel
+      char* const ent0 = smem + (kSlots == 2 ? (c & 1) * CS : 0) * SUB * kEntryBytes;
+      for (int i = copy_wave; i < kInstr * (HASZP ? 2 : 1); i += kCopyWaves) {
+        const bool is_zp = i >= kInstr;
+        const int ii = is_zp ? i - kInstr : i;
+        const int e = ii * kEpi + lane / kPieces, piece = lane % kPieces;
+        const int k_at = (c0 * SUB + e) * 128;
+        const int sblk = min(c_shift >= 0 ? (k_at >> c_shift) : k_at / C, n_sblk - 1);
+        int ch = n_wg0 + piece * (4 / SE);
+        if (ch + 4 / SE > N) ch = N - 4 / SE;    // channels past N: any valid address (never used)
+        const char* src = (const char*)(is_zp ? a.zp : a.scale) + ((size_t)sblk * N + ch) * SE;
+        char* dst = ent0 + (is_zp ? kSclTensor : 0) + ii * (kEpi * kEntryBytes);
+        __builtin_amdgcn_global_load_lds((const void*)src, (lds_ptr_t)dst, 4, 0, 0);
+      }
+    }
+    char* const slot = xsm + (kSlots == 2 ? (c & 1) * (CS * X_TILE) : 0);
     for (int row = copy_wave; row < x_rows; row += kCopyWaves) {
       const char* xrow = x_base + (size_t)row * ((size_t)ldk * XB) + (size_t)c0 * XROW;  // row `row`, first column of the chunk
       char* lrow = slot + row * XROW;
@@ -367,62 +411,53 @@ qmm_skinny_kernel(SkinnyArgs a) {
       });
     }
   };
-  // Blockwise: scale / zero point of 4 consecutive channels are one 16-byte
-  // load (8 of them used for 2-byte types), fetched one step ahead: bw_sc[t]
-  // holds those of the block that sub-step t of the current step lies in.
-  // (The entry point admits blockwise problems only with N % 4 == 0, for the
-  // alignment, at least 16 bytes of scales, and scales / zero points of x's
-  // dtype, as the reference's einsum requires: the conversions below are then
-  // free of run-time dtype branches.)
-  constexpr int kBw = RED == kRedRaw ? 1 : SUB;
-  i32x4 bw_sc[kBw], bw_zp[kBw];
-  int bw_sc_sel[kBw], bw_zp_sel[kBw];  // 2-byte types: 0 or 2, the dword pair of the load that holds the values
-  const int n_sblk = K / C;
-  const int c_shift = (C & (C - 1)) == 0 ? __builtin_ctz(C) : -1;  // block size a power of two: shift instead of divide
-  auto bw_fetch1 = [&](const void* base, int dt, int sblk, i32x4& dst, int& sel) __attribute__((always_inline)) {
-    const int esz = dt == XLA_AMD_DT_F32 ? 4 : 2;
-    const int64_t total = (int64_t)n_sblk * N * esz;
-    const int64_t off = ((int64_t)sblk * N + min(n_wave + 4 * g, N - 4)) * esz;
-    const int64_t at = min(off, total - 16);  // a 2-byte row end: read the 16 bytes that end there
-    sel = (int)(off - at) >> 2;
-    dst = *(const i32x4*)((const char*)base + at);
-  };
-  // scales of the block that sub-step t of this wave's s-th step lies in
-  auto bw_fetch = [&](int s, auto tc) __attribute__((always_inline)) {
+  // Blockwise: scale / zero point of this lane's 4 channels come from the entry of the sub-step
+  // that ends the block (x tile `ep_tile`, sub-step t), one LDS read each.
+  int ep_tile = 0;
+  auto bw_read = [&](int tensor, auto tc, float (&val)[4]) __attribute__((always_inline)) {
     constexpr int t = tc;
-    if constexpr (RED != kRedRaw) {
-      const int k_at = (s * KW + kw) * KS + t * 128;
-      const int sblk = min(c_shift >= 0 ? (k_at >> c_shift) : k_at / C, n_sblk - 1);
-      bw_fetch1(a.scale, XT, sblk, bw_sc[t], bw_sc_sel[t]);
-      if constexpr (HASZP) bw_fetch1(a.zp, XT, sblk, bw_zp[t], bw_zp_sel[t]);
+    const char* ent = smem + tensor * kSclTensor + (ep_tile * SUB + t) * kEntryBytes + (16 * rw + 4 * g) * SE;
+    if constexpr (SE == 4) {
+      const f32x4 r4 = *(const f32x4*)ent;
+      val[0] = r4[0]; val[1] = r4[1]; val[2] = r4[2]; val[3] = r4[3];
+    } else {
+      const i32x2 r2 = *(const i32x2*)ent;
+      val[0] = qmm_from_raw((uint32_t)r2[0] & 0xffffu, XT); val[1] = qmm_from_raw((uint32_t)r2[0] >> 16, XT);
+      val[2] = qmm_from_raw((uint32_t)r2[1] & 0xffffu, XT); val[3] = qmm_from_raw((uint32_t)r2[1] >> 16, XT);
     }
-  };
-  auto bw_value = [&](const i32x4& raw, int sel, int dt, auto vc) __attribute__((always_inline)) -> float {
-    constexpr int v = vc;
-    if (dt == XLA_AMD_DT_F32) return __int_as_float(raw[v]);
-    const uint32_t lo = (uint32_t)(sel ? raw[2] : raw[0]), hi = (uint32_t)(sel ? raw[3] : raw[1]);
-    const uint32_t dw = (v >> 1) ? hi : lo;
-    return qmm_from_raw((v & 1) ? (dw >> 16) : (dw & 0xffffu), dt);
   };
   auto block_epilogue = [&](int sblk, auto tc) __attribute__((always_inline)) {
     constexpr int t = tc;
+    float sc4[4], zp4[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (RED != kRedRaw) {
+      bw_read(0, tc, sc4);
+      if constexpr (HASZP) bw_read(1, tc, zp4);
+    }
+    // (every register of xs holds the row's sum: the lane's x row is the same for its 4 channels)
+    float xs_rounded[MT];
+    qmm_static_for<MT>([&](auto mc) { xs_rounded[(int)mc] = NEEDXS ? qmm_round_dt(xs[(int)mc][0], x_dt) : 0.f; });
     qmm_static_for<4>([&](auto vc) {
       constexpr int v = vc;
-      const int n = min(n_wave + 4 * g + v, N - 1);
       float sc, zv = 0.f;
       if constexpr (RED == kRedRaw) {
         sc = qmm_from_raw(pre_sc[v], scale_dt);
         if constexpr (HASZP) zv = qmm_from_raw(pre_zp[v], zp_dt);
       } else {
-        sc = bw_value(bw_sc[t], bw_sc_sel[t], XT, vc);
-        if constexpr (HASZP) zv = bw_value(bw_zp[t], bw_zp_sel[t], XT, vc);
+        sc = sc4[v];
+        zv = zp4[v];
       }
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
-        const float xsv = NEEDXS ? xs[mt][v] : 0.f;
-        const float p = qmm_round_dt(true_dot(acc[mt][v] + accb[mt][v], xsv), dot_dt);
+        const float xsv = NEEDXS ? xs[mt][0] : 0.f;
+        float p;
+        if constexpr (RED != kRedRaw && BITS == 4 && kMfma) {
+          // the int4 map's factor 16 is applied once, to the sum over the blocks (a power of two commutes with the rounding)
+          p = qmm_round_dt(fmaf(-1.5f, xsv, acc[mt][v] + accb[mt][v]), dot_dt);
+        } else {
+          p = qmm_round_dt(true_dot(acc[mt][v] + accb[mt][v], xsv), dot_dt);
+        }
         sacc[mt][v] = fmaf(sc, p, sacc[mt][v]);
-        if constexpr (HASZP) zacc[mt][v] = fmaf(qmm_round_dt(xsv, x_dt), zv, zacc[mt][v]);
+        if constexpr (HASZP) zacc[mt][v] = fmaf(xs_rounded[mt], zv, zacc[mt][v]);
       });
     });
     qmm_static_for<MT>([&](auto mc) {
@@ -449,7 +484,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
   auto compute = [&](auto pc, int tile, int s, auto refillc) __attribute__((always_inline)) {
     constexpr int p = pc;
     constexpr bool kRefill = refillc != 0;
-    const char* xb = smem + tile * X_TILE;
+    const char* xb = xsm + tile * X_TILE;
+    ep_tile = tile;
     const int k_step = (s * KW + kw) * KS;
     if constexpr (RED == kRedScaled) block_left = sub_per_block;  // steps start on block boundaries
     // x fragments of sub-step t: per tile of 16 x rows, this lane's XQ 16-byte chunks
@@ -532,7 +568,6 @@ qmm_skinny_kernel(SkinnyArgs a) {
         if (k_step + t * 128 < K) math(tc, wreg[p][kLoadsPerSub * t], wreg[p][kLoadsPerSub * t + kW1], xq[cur]);
         if constexpr (kRefill) {
           load_sub(pc, s + P, tc);
-          bw_fetch(s + 1, tc);
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -546,7 +581,6 @@ qmm_skinny_kernel(SkinnyArgs a) {
         }
         if constexpr (kRefill) {
           load_sub(pc, s + P, tc);
-          bw_fetch(s + 1, tc);
         }
       });
     }
@@ -566,13 +600,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // the compiler to wait for *all* outstanding loads wherever it needs one of
   // them.
   // First chunk: weights of step 0 are under way (issued at the top of the kernel) and so
-  // are the x copies; the first blockwise scales follow them.
-  qmm_static_for<kBw>([&](auto tc) { bw_fetch(0, tc); });
-  {
-    // vmcnt(kInFlight): everything older than the first scales has landed
-    constexpr int kInFlight = RED != kRedRaw ? (HASZP ? 2 : 1) * kBw : 0;
-    __builtin_amdgcn_s_waitcnt(((kInFlight >> 4) << 14) | 0x0F70 | (kInFlight & 15));
-  }
+  // are the x copies (with the blockwise scales of their sub-steps).
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first weights (and this wave's copies, if it copies) have landed
   qmm_bare_barrier();
   fetch_channel_scales();  // (per-channel) needed at the very end: their latency hides behind the main loop
   int s0 = 0;  // this wave's next step
@@ -682,8 +711,9 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const int m = 16 * mt + r;
     const int n = n_wave + 4 * g;
     if (m < M && n < N) {
-      float o0 = qmm_round_dt(sacc[mt][0], out_dt), o1 = qmm_round_dt(sacc[mt][1], out_dt);
-      float o2 = qmm_round_dt(sacc[mt][2], out_dt), o3 = qmm_round_dt(sacc[mt][3], out_dt);
+      constexpr float kBlockFactor = (RED != kRedRaw && BITS == 4 && kMfma) ? 16.0f : 1.0f;  // see block_epilogue
+      float o0 = qmm_round_dt(kBlockFactor * sacc[mt][0], out_dt), o1 = qmm_round_dt(kBlockFactor * sacc[mt][1], out_dt);
+      float o2 = qmm_round_dt(kBlockFactor * sacc[mt][2], out_dt), o3 = qmm_round_dt(kBlockFactor * sacc[mt][3], out_dt);
       if constexpr (HASZP) {
         o0 = qmm_round_dt(o0 - qmm_round_dt(zacc[mt][0], zpo_dt), out_dt);
         o1 = qmm_round_dt(o1 - qmm_round_dt(zacc[mt][1], zpo_dt), out_dt);
@@ -723,12 +753,13 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
     auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, UNI, NW, WSEG>;
     static std::atomic<uint64_t> lds_set{0};
     constexpr int kSlots = skinny_slots<Cfg, MT, RED, KW>();
-    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20, kSlots), lds_set, "weight_only_skinny hipFuncSetAttribute");
+    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20, kSlots) + skinny_scale_bytes<Cfg, XT, MT, RED, KW>(), lds_set, "weight_only_skinny hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
     const int steps = (a.k_per_slice + Cfg::KS - 1) / Cfg::KS;
+    constexpr int kScl = skinny_scale_bytes<Cfg, XT, MT, RED, KW>();
     hipLaunchKernelGGL(kern, dim3(blocks, (unsigned)a.slices), dim3((NW + skinny_copier_waves<MT, RED>()) * 64),
-                       Cfg::lds_bytes(steps, kSlots), stream, a);
+                       Cfg::lds_bytes(steps, kSlots) + kScl, stream, a);
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
