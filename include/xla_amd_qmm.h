@@ -159,7 +159,7 @@ int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const voi
  * Bytes of workspace xla_amd_qmm_weight_only_gemm needs for a shape (0 when it
  * needs none, or for arguments it rejects).
  */
-size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t C, int bits);
 
 /*
  * Weight-only quantized matmul for many rows of x (prefill-sized M), and for
@@ -170,10 +170,14 @@ size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_
  *   out = F.linear(x, w) * scaler;  out -= rowsum(x) (x) zp   (xla_quantized_matmul.py:113-114, :125-133)
  * and, with dot_dt = f32, the float branch of the Pallas kernel
  * (pallas_kernels/quantized_matmul_kernel.py:108-121).
- * Per-channel int8 weights only (w_tiled from xla_amd_qmm_tile_weight with
- * bits == 8), x [M,K] bf16 or f16, K % 128 == 0; other cases return
- * XLA_AMD_QMM_EUNSUPPORTED (the streaming kernel takes them).  dtype arguments
- * as for xla_amd_qmm_weight_only_skinny.  With at most 32 rows, few output
+ * x [M,K] bf16 or f16, w_tiled from xla_amd_qmm_tile_weight, K % 128 == 0; other
+ * cases return XLA_AMD_QMM_EUNSUPPORTED (the streaming kernel takes them).
+ * Per-channel int8 weights (C == K, bits == 8): dtype arguments as for
+ * xla_amd_qmm_weight_only_skinny.  Blockwise (C < K, C % 128 == 0) and int4
+ * weights (bits == 4): a tile of 64 rows x 128 channels with the rounding points
+ * of the blockwise statements (xla_quantized_matmul.py:115-133: every block's dot
+ * product rounded to x's dtype before it is scaled); scale / zp [K/C, N]; they
+ * need N % 4 == 0 and every dtype argument equal to x_dt, and use no workspace.  With at most 32 rows, few output
  * channels and a long K (where xla_amd_qmm_dispatch returns this kernel for such
  * an M) the call runs the streaming kernel over K slices instead, one slice of 64
  * channels per workgroup, and a second kernel adds the slices in slice order.
@@ -185,8 +189,8 @@ size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_
  */
 int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, const void* scale, const void* zp,
                                  void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
-                                 int64_t K, int x_dt, int scale_dt, int zp_dt, int dot_dt, int out_dt,
-                                 int store_dt, void* stream);
+                                 int64_t K, int64_t C, int bits, int x_dt, int scale_dt, int zp_dt, int dot_dt,
+                                 int out_dt, int store_dt, void* stream);
 
 /*
  * Weight-only quantized matmul for any shape, reading the operator's own

@@ -35,11 +35,11 @@ def wo_gemm(ops, x, w, s, z, dot_dtype=None, store_dtype=None):
   out_dtype = torch.promote_types(x.dtype, s.dtype)
   store_dtype = store_dtype or out_dtype
   out = torch.empty(m, n, dtype=store_dtype, device=x.device)
-  nbytes = lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k)
+  nbytes = lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k, k, 8)
   ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
   zp_dt = _lib.dt(z.dtype) if z is not None else _lib.dt(x.dtype)
   rc = lib.xla_amd_qmm_weight_only_gemm(x.data_ptr(), wt.data_ptr(), s.data_ptr(), _lib.ptr(z), out.data_ptr(), ws.data_ptr(),
-                                        nbytes, m, n, k, _lib.dt(x.dtype), _lib.dt(s.dtype), zp_dt,
+                                        nbytes, m, n, k, k, 8, _lib.dt(x.dtype), _lib.dt(s.dtype), zp_dt,
                                         _lib.dt(dot_dtype or x.dtype), _lib.dt(out_dtype), _lib.dt(store_dtype),
                                         torch.cuda.current_stream().cuda_stream)
   _lib.check(rc, "weight_only_gemm")
@@ -98,3 +98,37 @@ def test_weight_only_prefill_through_the_operator(ops):
   lin.load_quantized_weight(w.cuda(), s.cuda())
   x3 = x[:96].reshape(2, 48, k)
   check(lin(x3.cuda()), oracle.quantized_matmul(x3, w, s), "module, 3-D x")
+
+
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+def test_blockwise_and_int4_gemm(ops, xdt):
+  """More than 32 rows against blockwise or int4 weights: the tiled GEMM with per-block rounding points."""
+  op = torch.ops.xla.quantized_matmul
+  # (m, n, k, block, bits, asymmetric): one and several steps per block, block = chunk, row / channel tails,
+  # several chunks, more tiles than compute units
+  for (m, n, k, c, bits, asym) in [(65, 128, 256, 128, 8, False), (100, 200, 1024, 128, 4, True), (128, 4096, 4096, 128, 4, True),
+                                   (130, 60, 1536, 512, 8, True), (300, 1000, 2048, 256, 4, False), (65, 4, 128, 128, 4, True),
+                                   (70, 132, 2560, 640, 8, False), (513, 8192, 1024, 128, 4, True)]:
+    x, w, s, z, _ = cases.blockwise(m, n, k, c, bits, xdt, symmetric=not asym, seed=m + n)
+    exp = oracle.quantized_matmul(x, w, s, z if asym else None, block_size=c, int4_weight=bits == 4)
+    before = ops.counters["wo_gemm"]
+    out = op(x.cuda(), w.cuda(), s.cuda(), z.cuda() if asym else None, c, bits == 4)
+    assert ops.counters["wo_gemm"] == before + 1
+    rl2 = check(out, exp, f"blockwise GEMM {m, n, k, c, bits, asym, xdt}")
+    assert rl2 < 1e-3, (m, n, k, c, bits, rl2)
+  # per-channel int4 (one block)
+  for (m, n, k, zp) in [(77, 512, 1024, False), (200, 100, 384, True)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m)
+    w = w.clamp(-8, 7)
+    z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(xdt) if zp else None
+    exp = oracle.quantized_matmul(x, w, s, z, int4_weight=True)
+    before = ops.counters["wo_gemm"]
+    out = op(x.cuda(), w.cuda(), s.cuda(), None if z is None else z.cuda(), -1, True)
+    assert ops.counters["wo_gemm"] == before + 1
+    check(out, exp, f"per-channel int4 GEMM {m, n, k, zp, xdt}")
+  # mixed dtypes (f32 scale with 2-byte x) keep the streaming kernel
+  x, w, s, _ = cases.per_channel_int8(80, 64, 256, xdt, torch.float32, seed=9)
+  before = ops.counters["skinny_mfma"]
+  out = op(x.cuda(), w.clamp(-8, 7).cuda(), s.cuda(), None, -1, True)
+  assert ops.counters["skinny_mfma"] == before + 1
+  check(out, oracle.quantized_matmul(x, w.clamp(-8, 7), s, int4_weight=True), "int4, f32 scale")

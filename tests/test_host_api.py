@@ -57,14 +57,18 @@ def test_dispatcher_regimes():
   assert d(33, 14336, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F32, 0) == _lib.KERNEL_SKINNY_MFMA
-  assert d(2048, 4096, 4096, 128, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # blockwise
-  assert d(2048, 14336, 4096, 4096, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA    # int4
+  assert d(2048, 4096, 4096, 128, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # blockwise: its own tiled GEMM
+  assert d(2048, 14336, 4096, 4096, 4, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # int4 too
+  assert d(64, 4096, 4096, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA         # up to 64 rows stream (two passes)
+  assert d(2048, 4096, 4096, 128, 4, _lib.DT_F32, 0) == _lib.KERNEL_SKINNY_MFMA        # f32 x: no GEMM
+  assert d(100, 30, 256, 128, 8, _lib.DT_BF16, 0) == _lib.KERNEL_GENERIC               # blockwise needs N % 4 == 0
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 4096, 4096, 128, 4) == 0
   assert d(32, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(4, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # too few rows of x to matter
   assert d(32, 4096, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA       # K too short for slices
   assert d(32, 14336, 8192, 8192, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # enough workgroups already
-  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336) == 4 * (32 * 4096 + 32) * 4  # four K slices
-  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 14336, 4096) == 0
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336, 14336, 8) == 4 * (32 * 4096 + 32) * 4  # four K slices
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 14336, 4096, 4096, 8) == 0
   assert d(2048, 14336, 4096, 4096, 8, _lib.DT_BF16, 1) == _lib.KERNEL_W8A8_MFMA
   assert d(3, 8, 5, 5, 8, _lib.DT_F32, 1) == _lib.KERNEL_W8A8_GENERIC
   tile = (ctypes.c_int32 * 3)()

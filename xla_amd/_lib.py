@@ -33,8 +33,8 @@ SIGNATURES = {
     "xla_amd_qmm_tile_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
     "xla_amd_qmm_untile_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
     "xla_amd_qmm_weight_only_skinny": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),
-    "xla_amd_qmm_weight_only_gemm_workspace_bytes": (ctypes.c_size_t, [_c_i64] * 3),
-    "xla_amd_qmm_weight_only_gemm": (_c_int, [_c_vp] * 6 + [ctypes.c_size_t] + [_c_i64] * 3 + [_c_int] * 6 + [_c_vp]),
+    "xla_amd_qmm_weight_only_gemm_workspace_bytes": (ctypes.c_size_t, [_c_i64] * 4 + [_c_int]),
+    "xla_amd_qmm_weight_only_gemm": (_c_int, [_c_vp] * 6 + [ctypes.c_size_t] + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),
     "xla_amd_qmm_weight_only_generic": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),
     "xla_amd_qmm_quantize_per_token": (_c_int, [_c_vp] * 4 + [_c_i64] * 2 + [_c_int] * 3 + [_c_vp]),
     "xla_amd_qmm_w8a8_gemm": (_c_int, [_c_vp] * 8 + [_c_i64] * 3 + [_c_int] * 9 + [_c_vp]),

@@ -94,6 +94,13 @@ extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, 
     int per;
     if (M > 32 || qmm_skinny_k_slices(M, N, K, &per) > 1) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
   }
+  // many rows against blockwise or int4 weights: the tiled GEMM with per-block rounding points (the caller
+  // must also have scale / zero point / result of x's dtype; else it takes the streaming kernel, pass by pass).
+  // Up to 64 rows two passes of the streaming kernel are as fast or faster (a 64 x 128 tile per workgroup and
+  // no K split: 4096 channels are 32 workgroups).
+  if ((C != K || bits == 4) && (bits == 8 || bits == 4) && K % 128 == 0 && C % 128 == 0 && N % 4 == 0 &&
+      x_dt != XLA_AMD_DT_F32 && M > 64)
+    return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
   if (K % 128 == 0 && C % 128 == 0 && (bits == 8 || bits == 4) && M >= 1 &&
       (C == K || (N % 4 == 0 && (K / C) * N >= 8)))  // blockwise: vector loads of 4 channels' scales
     return XLA_AMD_KERNEL_SKINNY_MFMA;

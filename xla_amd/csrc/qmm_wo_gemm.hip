@@ -33,7 +33,9 @@
 // -DQMM_WO_MT=4|8) so that the units build in parallel; the unit of bf16 with MT = 8 also
 // holds the second kernel of a K split and the C entry points.
 #include "qmm_common.h"
+#include "qmm_frag.h"
 #include "qmm_skinny.h"
+#include "qmm_wo_bw.h"
 
 #if !defined(QMM_WO_XT) || !defined(QMM_WO_MT)
 #error "compile with -DQMM_WO_XT=<XLA_AMD_DT_BF16|XLA_AMD_DT_F16 value> -DQMM_WO_MT=<4|8>"
@@ -65,45 +67,7 @@ constexpr int kComputeWaves = 4;
 constexpr int kCopyWaves = 4;
 constexpr int kLds = 160 * 1024;
 
-__device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
-  // {bf16(lo), bf16(hi)} by truncation: exact for integers of magnitude <= 256.
-  return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
-}
-__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
-  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-  h2 v = __builtin_bit_cast(h2, __builtin_amdgcn_cvt_pkrtz(lo, hi));  // exact for small integers
-  return __builtin_bit_cast(uint32_t, v);
-}
-// 8 int8 weights (two dwords) -> 8 elements of the x dtype.
-template <int XT>
-__device__ __forceinline__ i32x4 cvt_w8(uint32_t d0, uint32_t d1) {
-  float f[8];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    f[i] = (float)(int8_t)(d0 >> (8 * i));
-    f[4 + i] = (float)(int8_t)(d1 >> (8 * i));
-  }
-  i32x4 o;
-  if constexpr (XT == XLA_AMD_DT_BF16) {
-    o[0] = pack_hi16(f[0], f[1]); o[1] = pack_hi16(f[2], f[3]);
-    o[2] = pack_hi16(f[4], f[5]); o[3] = pack_hi16(f[6], f[7]);
-  } else {
-    o[0] = pack_f16(f[0], f[1]); o[1] = pack_f16(f[2], f[3]);
-    o[2] = pack_f16(f[4], f[5]); o[3] = pack_f16(f[6], f[7]);
-  }
-  return o;
-}
-template <int XT>
-__device__ __forceinline__ f32x4 mfma16(i32x4 a, i32x4 b, f32x4 c) {
-  if constexpr (XT == XLA_AMD_DT_BF16)
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  else
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-}
-template <int XT> __device__ __forceinline__ i32x4 ones_frag() {
-  const uint32_t one2 = XT == XLA_AMD_DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
-  return i32x4{(int)one2, (int)one2, (int)one2, (int)one2};
-}
+using namespace qmm_frag;
 
 template <int MT> struct WoCfg {
   static constexpr int BM = 16 * MT;
@@ -537,8 +501,10 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
 
 }  // namespace
 
-extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t C, int bits) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  if (C <= 0) C = K;
+  if (C != K || bits != 8) return 0;  // blockwise / int4 weights: no K split, no workspace
   if (M <= 32) {  // the weight-streaming kernel over K slices
     int per;
     const int slices = qmm_skinny_k_slices(M, N, K, &per);
@@ -557,11 +523,32 @@ extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_
 
 extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, const void* scale, const void* zp,
                                             void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
-                                            int64_t K, int x_dt, int scale_dt, int zp_dt, int dot_dt, int out_dt,
-                                            int store_dt, void* stream) {
+                                            int64_t K, int64_t C, int bits, int x_dt, int scale_dt, int zp_dt,
+                                            int dot_dt, int out_dt, int store_dt, void* stream) {
   if (!x || !w_tiled || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: null pointer");
-  if (M < 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad sizes M=%lld N=%lld K=%lld",
-                                                 (long long)M, (long long)N, (long long)K);
+  if (M < 0 || N <= 0 || K <= 0 || C <= 0 || K % C != 0)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad sizes M=%lld N=%lld K=%lld C=%lld", (long long)M,
+                    (long long)N, (long long)K, (long long)C);
+  if (bits != 4 && bits != 8) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bits must be 4 or 8");
+  if (C != K || bits != 8) {
+    // blockwise and int4 weights: the tiled GEMM with per-block rounding points (every dtype x's)
+    if (!qmm_valid_dt(x_dt) || x_dt == XLA_AMD_DT_F32)
+      return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x must be bf16 or f16");
+    if (scale_dt != x_dt || (zp && zp_dt != x_dt) || dot_dt != x_dt || out_dt != x_dt || store_dt != x_dt)
+      return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: blockwise / int4 weights need every dtype to be x's");
+    if (K % 128 != 0 || C % 128 != 0 || N % 4 != 0)
+      return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: blockwise / int4 weights need K %% 128 == 0, C %% 128 == 0, N %% 4 == 0");
+    if (N > (1 << 30) || K > (1 << 24) || M > (1 << 24))
+      return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: dimension too large");
+    if ((((uintptr_t)x | (uintptr_t)w_tiled) & 15) || ((uintptr_t)out & 7) || ((uintptr_t)scale & 3) || ((uintptr_t)zp & 3))
+      return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x and w must be 16-byte, out 8-byte, scale / zero point 4-byte aligned");
+    if (M == 0) return XLA_AMD_QMM_OK;
+    WoBwArgs b;
+    b.x = x; b.w = (const uint8_t*)w_tiled; b.scale = scale; b.zp = zp; b.out = out;
+    b.M = (int)M; b.N = (int)N; b.K = (int)K; b.C = (int)C;
+    return x_dt == XLA_AMD_DT_BF16 ? qmm_wo_bw_launch_bf16(b, bits, (hipStream_t)stream)
+                                   : qmm_wo_bw_launch_f16(b, bits, (hipStream_t)stream);
+  }
   if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || !qmm_valid_dt(dot_dt) ||
       !qmm_valid_dt(store_dt) || (zp && !qmm_valid_dt(zp_dt)))
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad dtype enum");

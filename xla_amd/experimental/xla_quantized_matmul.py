@@ -219,14 +219,20 @@ def _weight_only_launch(x2, w, w_tiled, n, k, c, layout, bits, scaler, zero_poin
   zp_dt = _lib.dt(zero_point.dtype) if zero_point is not None else _lib.dt(x2.dtype)
   dts = (_lib.dt(x2.dtype), _lib.dt(scaler.dtype), zp_dt, _lib.dt(dot_dtype), _lib.dt(out_dtype),
          _lib.dt(store_dtype))
+  if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM and (c != k or bits == 4):
+    # the tiled GEMM for blockwise / int4 weights computes in one dtype throughout
+    same = (scaler.dtype == x2.dtype and (zero_point is None or zero_point.dtype == x2.dtype) and
+            dot_dtype == x2.dtype and out_dtype == x2.dtype and store_dtype == x2.dtype)
+    if not same:
+      kern = _lib.KERNEL_SKINNY_MFMA
   if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM:
     wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
     counters["wo_gemm"] += 1
-    nbytes = lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k)
+    nbytes = lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k, c, bits)
     workspace = torch.empty(nbytes, dtype=torch.uint8, device=x2.device) if nbytes else None
     _lib.check(
         lib.xla_amd_qmm_weight_only_gemm(x2.data_ptr(), wk.data_ptr(), scaler.data_ptr(), _lib.ptr(zero_point),
-                                         out.data_ptr(), _lib.ptr(workspace), nbytes, m, n, k, *dts, stream),
+                                         out.data_ptr(), _lib.ptr(workspace), nbytes, m, n, k, c, bits, *dts, stream),
         "weight_only_gemm")
   elif kern == _lib.KERNEL_SKINNY_MFMA:
     wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
