@@ -194,7 +194,17 @@ def main():
     extra["blockwise_int4_M16"] = {"us": round(ev * 1e3, 3), "GBps": round(b3 / ev / 1e6, 1),
                                    "frac_hbm": round(b3 / ev / 1e6 / HBM_PEAK_GBPS, 4),
                                    "algorithmic_bytes": b3}
-    del w3s, fns
+    # the same weights against a prefill-sized M: the tiled GEMM with per-block rounding points
+    x3p = torch.randn(2048, 4096, generator=cases.gen(4)).bfloat16().to(dev)
+    w3d = w3s[0]
+    _, ev, _ = time_calls([lambda: op(x3p, w3d, s3d, z3d, block_size=128, int4_weight=True)], 20, 5, use_graph)
+    f3 = 2.0 * 2048 * 4096 * 4096
+    extra["blockwise_int4_prefill_M2048"] = {
+        "us": round(ev * 1e3, 2),
+        "roofline": {"bound": "mfma", "achieved": round(f3 / ev / 1e9, 1), "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(f3 / ev / 1e9 / BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "qmm_wo_bw_gemm_kernel<bf16, int4, zero point> (64 x 128 tiles)"}}
+    del w3s, fns, x3p, w3d
 
     # W8A8 prefill GEMM (config 4)
     m4 = 2048
