@@ -132,3 +132,18 @@ def test_blockwise_and_int4_gemm(ops, xdt):
   out = op(x.cuda(), w.clamp(-8, 7).cuda(), s.cuda(), None, -1, True)
   assert ops.counters["skinny_mfma"] == before + 1
   check(out, oracle.quantized_matmul(x, w.clamp(-8, 7), s, int4_weight=True), "int4, f32 scale")
+
+
+@pytest.mark.parametrize("zp", [False, True])
+def test_int4_per_channel_k_slices(ops, zp):
+  """Few rows, few channels, long K with per-channel int4 weights: the streaming kernel over K slices (steps of 1024 columns)."""
+  op = torch.ops.xla.quantized_matmul
+  for (m, n, k, sdt) in [(32, 4096, 14336, torch.bfloat16), (9, 1000, 8192, torch.bfloat16), (16, 2048, 10240, torch.float32)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, torch.bfloat16, sdt, seed=n)
+    w = w.clamp(-8, 7)
+    z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(sdt) if zp else None
+    exp = oracle.quantized_matmul(x, w, s, z, int4_weight=True)
+    before = ops.counters["wo_gemm"]
+    out = op(x.cuda(), w.cuda(), s.cuda(), None if z is None else z.cuda(), -1, True)
+    assert ops.counters["wo_gemm"] == before + 1
+    check(out, exp, f"int4 K slices {m, n, k, sdt, zp}")

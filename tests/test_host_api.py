@@ -63,6 +63,9 @@ def test_dispatcher_regimes():
   assert d(2048, 4096, 4096, 128, 4, _lib.DT_F32, 0) == _lib.KERNEL_SKINNY_MFMA        # f32 x: no GEMM
   assert d(100, 30, 256, 128, 8, _lib.DT_BF16, 0) == _lib.KERNEL_GENERIC               # blockwise needs N % 4 == 0
   assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 4096, 4096, 128, 4) == 0
+  assert d(32, 4096, 14336, 14336, 4, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # int4 K slices (steps of 1024 columns)
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336, 14336, 4) == 4 * (32 * 4096 + 32) * 4
+  assert d(32, 4096, 14336, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA          # blockwise: no K slices
   assert d(32, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(4, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # too few rows of x to matter
   assert d(32, 4096, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA       # K too short for slices

@@ -14,8 +14,8 @@ struct SkinnyArgs {
   int scale_dt, zp_dt, out_dt;
   int dot_dt;    // dtype the dot product is rounded to before it is scaled (per-channel only)
   int store_dt;  // dtype of the stored tensor (out_dt, or a final cast of it)
-  // K slices over workgroups (per-channel int8 only): blockIdx.y = slice of k_per_slice columns (a
-  // multiple of 512; K when there is one slice).  With slices the kernel stores its raw sums instead
+  // K slices over workgroups (per-channel weights only): blockIdx.y = slice of k_per_slice columns (a
+  // multiple of the kernel's step, 512 columns for int8 and 1024 for int4; K when there is one slice).  With slices the kernel stores its raw sums instead
   // of results: part [slices][M][N] dot products, part_xs [slices][M] row sums of x (zero point only).
   int k_per_slice;
   int slices;
@@ -27,6 +27,6 @@ int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t
 int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
 int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
 
-// K slices the streaming kernel should run a per-channel int8 launch of M <= 32 rows in (1 = none):
+// K slices the streaming kernel should run a per-channel launch of M <= 32 rows in (1 = none):
 // few output channels against a long K, where every workgroup would otherwise copy all of x.
-int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int* k_per_slice);
+int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int bits, int* k_per_slice);

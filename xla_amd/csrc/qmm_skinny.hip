@@ -626,7 +626,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
         const int n = n_wave + 4 * g;
         if (m < M && n < N) {
           float* p = a.part + ((size_t)slice * M + m) * N + n;
-          const f32x4 t = {acc[mt][0] + accb[mt][0], acc[mt][1] + accb[mt][1], acc[mt][2] + accb[mt][2], acc[mt][3] + accb[mt][3]};
+          // (the slice's dot product: with int4 weights the affine map is undone with the slice's own row sum)
+          const float xsv = NEEDXS ? xs[mt][0] : 0.f;
+          const f32x4 t = {true_dot(acc[mt][0] + accb[mt][0], xsv), true_dot(acc[mt][1] + accb[mt][1], xsv),
+                           true_dot(acc[mt][2] + accb[mt][2], xsv), true_dot(acc[mt][3] + accb[mt][3], xsv)};
           if ((N & 3) == 0) *(f32x4*)p = t;
           else for (int v = 0; v < 4; ++v) if (n + v < N) p[v] = t[v];
           if constexpr (NEEDXS) {

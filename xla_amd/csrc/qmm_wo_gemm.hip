@@ -504,12 +504,12 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
 extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t C, int bits) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
   if (C <= 0) C = K;
-  if (C != K || bits != 8) return 0;  // blockwise / int4 weights: no K split, no workspace
-  if (M <= 32) {  // the weight-streaming kernel over K slices
+  if (C == K && M <= 32) {  // the weight-streaming kernel over K slices
     int per;
-    const int slices = qmm_skinny_k_slices(M, N, K, &per);
+    const int slices = qmm_skinny_k_slices(M, N, K, bits, &per);
     if (slices > 1) return ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
   }
+  if (C != K || bits != 8) return 0;  // blockwise / int4 weights: the tiled GEMM splits no K and needs no workspace
   size_t need = 0;
   for (int zp = 0; zp < 2; ++zp) {  // the larger of the two plans: the size does not depend on the zero point
     const Plan p = make_plan(M, N, K, zp != 0);
@@ -530,6 +530,49 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad sizes M=%lld N=%lld K=%lld C=%lld", (long long)M,
                     (long long)N, (long long)K, (long long)C);
   if (bits != 4 && bits != 8) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bits must be 4 or 8");
+  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || !qmm_valid_dt(dot_dt) ||
+      !qmm_valid_dt(store_dt) || (zp && !qmm_valid_dt(zp_dt)))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad dtype enum");
+  if (out_dt != qmm_promote(x_dt, scale_dt))
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: out dtype must be promote(x, scale)");
+  if (dot_dt != x_dt && dot_dt != XLA_AMD_DT_F32)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: dot dtype must be x's or f32");
+  if (x_dt == XLA_AMD_DT_F32) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x must be bf16 or f16");
+  if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: K=%lld must be a multiple of 128", (long long)K);
+  if (N > (1 << 30) || K > (1 << 24) || M > (1 << 24))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: dimension too large");
+  if (((uintptr_t)x | (uintptr_t)w_tiled) & 15)
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x and w must be 16-byte aligned");
+  if (((uintptr_t)out & 15) && (N & 3) == 0)
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: out must be 16-byte aligned");
+  if (M == 0) return XLA_AMD_QMM_OK;
+  if (C == K && M <= 32) {
+    // few rows: the weight-streaming kernel over K slices, when that is what its plan says and the workspace is there
+    int per;
+    const int slices = qmm_skinny_k_slices(M, N, K, bits, &per);
+    const size_t need = ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
+    if (slices > 1 && workspace && workspace_bytes >= need && (((uintptr_t)workspace) & 15) == 0) {
+      SkinnyArgs k;
+      k.x = x; k.w = (const uint8_t*)w_tiled; k.scale = scale; k.zp = zp; k.out = out;
+      k.M = (int)M; k.N = (int)N; k.K = (int)K; k.C = (int)K;
+      k.scale_dt = scale_dt; k.zp_dt = zp ? zp_dt : x_dt; k.out_dt = out_dt; k.dot_dt = dot_dt; k.store_dt = store_dt;
+      k.k_per_slice = per; k.slices = slices;
+      k.part = (float*)workspace;
+      k.part_xs = k.part + (size_t)slices * (size_t)M * (size_t)N;
+      int rc = x_dt == XLA_AMD_DT_BF16 ? qmm_skinny_launch_bf16(k, bits, zp != nullptr, (hipStream_t)stream)
+                                       : qmm_skinny_launch_f16(k, bits, zp != nullptr, (hipStream_t)stream);
+      if (rc != XLA_AMD_QMM_OK) return rc;
+      WoGemmArgs f;
+      f.x = x; f.w = (const uint8_t*)w_tiled; f.scale = scale; f.zp = zp; f.out = out;
+      f.part = k.part; f.part_xs = k.part_xs;
+      f.M = (int)M; f.N = (int)N; f.K = (int)K; f.k_per_split = per; f.split = slices;
+      f.scale_dt = scale_dt; f.zp_dt = zp ? zp_dt : x_dt; f.dot_dt = dot_dt; f.out_dt = out_dt; f.store_dt = store_dt;
+      const int64_t threads = M * ((N + 3) / 4);
+      hipLaunchKernelGGL(qmm_wo_gemm_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                         (hipStream_t)stream, f, x_dt);
+      return QMM_CHECK_LAUNCH("weight_only_gemm finish launch");
+    }
+  }
   if (C != K || bits != 8) {
     // blockwise and int4 weights: the tiled GEMM with per-block rounding points (every dtype x's)
     if (!qmm_valid_dt(x_dt) || x_dt == XLA_AMD_DT_F32)
@@ -548,49 +591,6 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
     b.M = (int)M; b.N = (int)N; b.K = (int)K; b.C = (int)C;
     return x_dt == XLA_AMD_DT_BF16 ? qmm_wo_bw_launch_bf16(b, bits, (hipStream_t)stream)
                                    : qmm_wo_bw_launch_f16(b, bits, (hipStream_t)stream);
-  }
-  if (!qmm_valid_dt(x_dt) || !qmm_valid_dt(scale_dt) || !qmm_valid_dt(out_dt) || !qmm_valid_dt(dot_dt) ||
-      !qmm_valid_dt(store_dt) || (zp && !qmm_valid_dt(zp_dt)))
-    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: bad dtype enum");
-  if (out_dt != qmm_promote(x_dt, scale_dt))
-    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: out dtype must be promote(x, scale)");
-  if (dot_dt != x_dt && dot_dt != XLA_AMD_DT_F32)
-    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: dot dtype must be x's or f32");
-  if (x_dt == XLA_AMD_DT_F32) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x must be bf16 or f16");
-  if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: K=%lld must be a multiple of 128", (long long)K);
-  if (N > (1 << 30) || K > (1 << 24) || M > (1 << 24))
-    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: dimension too large");
-  if (((uintptr_t)x | (uintptr_t)w_tiled) & 15)
-    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x and w must be 16-byte aligned");
-  if (((uintptr_t)out & 15) && (N & 3) == 0)
-    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: out must be 16-byte aligned");
-  if (M == 0) return XLA_AMD_QMM_OK;
-  if (M <= 32) {
-    // few rows: the weight-streaming kernel over K slices, when that is what its plan says and the workspace is there
-    int per;
-    const int slices = qmm_skinny_k_slices(M, N, K, &per);
-    const size_t need = ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
-    if (slices > 1 && workspace && workspace_bytes >= need && (((uintptr_t)workspace) & 15) == 0) {
-      SkinnyArgs k;
-      k.x = x; k.w = (const uint8_t*)w_tiled; k.scale = scale; k.zp = zp; k.out = out;
-      k.M = (int)M; k.N = (int)N; k.K = (int)K; k.C = (int)K;
-      k.scale_dt = scale_dt; k.zp_dt = zp ? zp_dt : x_dt; k.out_dt = out_dt; k.dot_dt = dot_dt; k.store_dt = store_dt;
-      k.k_per_slice = per; k.slices = slices;
-      k.part = (float*)workspace;
-      k.part_xs = k.part + (size_t)slices * (size_t)M * (size_t)N;
-      int rc = x_dt == XLA_AMD_DT_BF16 ? qmm_skinny_launch_bf16(k, 8, zp != nullptr, (hipStream_t)stream)
-                                       : qmm_skinny_launch_f16(k, 8, zp != nullptr, (hipStream_t)stream);
-      if (rc != XLA_AMD_QMM_OK) return rc;
-      WoGemmArgs f;
-      f.x = x; f.w = (const uint8_t*)w_tiled; f.scale = scale; f.zp = zp; f.out = out;
-      f.part = k.part; f.part_xs = k.part_xs;
-      f.M = (int)M; f.N = (int)N; f.K = (int)K; f.k_per_split = per; f.split = slices;
-      f.scale_dt = scale_dt; f.zp_dt = zp ? zp_dt : x_dt; f.dot_dt = dot_dt; f.out_dt = out_dt; f.store_dt = store_dt;
-      const int64_t threads = M * ((N + 3) / 4);
-      hipLaunchKernelGGL(qmm_wo_gemm_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
-                         (hipStream_t)stream, f, x_dt);
-      return QMM_CHECK_LAUNCH("weight_only_gemm finish launch");
-    }
   }
   const Plan p = make_plan(M, N, K, zp != nullptr);
   WoGemmArgs a;

@@ -219,7 +219,7 @@ def _weight_only_launch(x2, w, w_tiled, n, k, c, layout, bits, scaler, zero_poin
   zp_dt = _lib.dt(zero_point.dtype) if zero_point is not None else _lib.dt(x2.dtype)
   dts = (_lib.dt(x2.dtype), _lib.dt(scaler.dtype), zp_dt, _lib.dt(dot_dtype), _lib.dt(out_dtype),
          _lib.dt(store_dtype))
-  if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM and (c != k or bits == 4):
+  if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM and (c != k or bits == 4) and m > 32:
     # the tiled GEMM for blockwise / int4 weights computes in one dtype throughout
     same = (scaler.dtype == x2.dtype and (zero_point is None or zero_point.dtype == x2.dtype) and
             dot_dtype == x2.dtype and out_dtype == x2.dtype and store_dtype == x2.dtype)
