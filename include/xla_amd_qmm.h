@@ -177,15 +177,19 @@ size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_
  * weights (bits == 4): a tile of 64 rows x 128 channels with the rounding points
  * of the blockwise statements (xla_quantized_matmul.py:115-133: every block's dot
  * product rounded to x's dtype before it is scaled); scale / zp [K/C, N]; they
- * need N % 4 == 0 and every dtype argument equal to x_dt, and use no workspace.  With at most 32 rows, few output
- * channels and a long K (where xla_amd_qmm_dispatch returns this kernel for such
- * an M) the call runs the streaming kernel over K slices instead, one slice of 64
- * channels per workgroup, and a second kernel adds the slices in slice order.
- * When K is split over workgroups the
- * partial sums live in `workspace` (device memory of at least
- * xla_amd_qmm_weight_only_gemm_workspace_bytes(M, N, K) bytes, 16-byte
- * aligned, free again when the call's work has completed); it may be NULL
- * when that size is 0.
+ * need N % 4 == 0 and every dtype argument equal to x_dt, and use no workspace.
+ * With at most 32 rows, few output channels and a long K (where
+ * xla_amd_qmm_dispatch returns this kernel for such an M) the call runs the
+ * streaming kernel over K slices instead, one slice of 64 channels per
+ * workgroup, and a second kernel adds the slices in slice order; slices of
+ * blockwise weights are whole quantization blocks, and what is added are the
+ * blocks' scaled, rounded dot products (and zero-point terms), so the rounding
+ * points stay the reference's.
+ * When K is split over workgroups the partial sums live in `workspace`
+ * (device memory of at least
+ * xla_amd_qmm_weight_only_gemm_workspace_bytes(M, N, K, C, bits) bytes,
+ * 16-byte aligned, free again when the call's work has completed); it may be
+ * NULL when that size is 0.
  */
 int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, const void* scale, const void* zp,
                                  void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,

@@ -147,3 +147,24 @@ def test_int4_per_channel_k_slices(ops, zp):
     out = op(x.cuda(), w.cuda(), s.cuda(), None if z is None else z.cuda(), -1, True)
     assert ops.counters["wo_gemm"] == before + 1
     check(out, exp, f"int4 K slices {m, n, k, sdt, zp}")
+
+
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+def test_blockwise_k_slices(ops, xdt):
+  """Few rows, few channels, long K with blockwise weights: K slices of whole quantization blocks; the second kernel adds
+  the slices' scaled sums (and zero-point sums) and does the final roundings."""
+  op = torch.ops.xla.quantized_matmul
+  lib = _lib.load()
+  # (m, n, k, block, bits, asymmetric): blocks shorter than, equal to and longer than a step of the streaming kernel
+  # (512 columns of int8, 1024 of int4), a last slice shorter than the others, row tails, one and two row tiles
+  for (m, n, k, c, bits, asym) in [(32, 4096, 14336, 128, 4, True), (16, 4096, 14336, 128, 8, False), (9, 1000, 8192, 256, 4, True),
+                                   (32, 2048, 14336, 2048, 8, True), (24, 512, 10240, 1024, 4, False), (8, 64, 16384, 512, 8, True),
+                                   (32, 200, 8192, 128, 4, True)]:
+    assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k, c, bits) > 0, (m, n, k, c, bits)
+    x, w, s, z, _ = cases.blockwise(m, n, k, c, bits, xdt, symmetric=not asym, seed=m + n)
+    exp = oracle.quantized_matmul(x, w, s, z if asym else None, block_size=c, int4_weight=bits == 4)
+    before = ops.counters["wo_gemm"]
+    out = op(x.cuda(), w.cuda(), s.cuda(), z.cuda() if asym else None, c, bits == 4)
+    assert ops.counters["wo_gemm"] == before + 1
+    rl2 = check(out, exp, f"blockwise K slices {m, n, k, c, bits, asym, xdt}")
+    assert rl2 < 1e-3, (m, n, k, c, bits, rl2)

@@ -65,7 +65,11 @@ def test_dispatcher_regimes():
   assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 4096, 4096, 128, 4) == 0
   assert d(32, 4096, 14336, 14336, 4, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # int4 K slices (steps of 1024 columns)
   assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336, 14336, 4) == 4 * (32 * 4096 + 32) * 4
-  assert d(32, 4096, 14336, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA          # blockwise: no K slices
+  assert d(32, 4096, 14336, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM     # blockwise K slices (whole blocks)
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336, 128, 4) == 2 * 4 * 32 * 4096 * 4  # sums + zero-point sums
+  assert d(32, 4096, 14336, 7168, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA         # a slice is whole blocks, at least two of them: two blocks stay one slice
+  assert d(32, 4098, 14336, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_GENERIC              # blockwise needs N % 4 == 0
+  assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336, 2048, 8) == 2 * 3 * 32 * 4096 * 4  # 3 + 3 + 1 blocks
   assert d(32, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(4, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # too few rows of x to matter
   assert d(32, 4096, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA       # K too short for slices

@@ -54,16 +54,22 @@ extern "C" size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits) {
 //    byte, so the weight is streamed exactly once by the skinny kernel;
 //  * many rows with int8 activations (prefill): LDS-tiled int8 MFMA GEMM.
 // Shapes neither fast kernel accepts run the one-thread-per-output kernels.
-// K slices over workgroups for the weight-streaming kernel (per-channel weights, int8 or int4).  A workgroup of that kernel owns 64
+// K slices over workgroups for the weight-streaming kernel.  A workgroup of that kernel owns 64
 // (or 32, 16) output channels over all of K and copies every column of x it multiplies; with few
 // channels and a long K the workgroups together copy several times the weight's bytes of x (out
 // of L2), and there are too few of them for the memory system.  Slicing K gives each workgroup
 // 64 channels of one slice: as many workgroups, a fraction of the x traffic.  The slices' sums are
 // added by a second kernel, so this needs a workspace and is reached through
 // xla_amd_qmm_weight_only_gemm.
-int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int bits, int* k_per_slice) {
+int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int64_t C, int bits, int* k_per_slice) {
   *k_per_slice = (int)K;
-  const int64_t ks = bits == 4 ? 1024 : 512;  // columns per step of the streaming kernel
+  int64_t ks = bits == 4 ? 1024 : 512;  // columns per step of the streaming kernel
+  if (C > 0 && C < K) {
+    // blockwise weights: a slice is whole steps and whole quantization blocks
+    if (C % 128 != 0 || K % C != 0 || N % 4 != 0) return 1;
+    if (C > ks) { if (C % ks != 0) return 1; ks = C; }
+    else if (ks % C != 0) return 1;
+  }
   if (M > 32 || K % ks != 0) return 1;
   // (measured with cold weights at M = 32: 4096 x 14336 25.5 -> 17.8 us; with K = 4096 or fewer than 8 rows the
   // second kernel costs more than the copies saved)
@@ -92,9 +98,9 @@ extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, 
   // many rows of 2-byte x against per-channel int8 weights: the tiled GEMM reads the weight once
   // per 128 rows, the streaming kernel once per 32
   if (C == K && bits == 8 && K % 128 == 0 && x_dt != XLA_AMD_DT_F32 && M > 32) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
-  if (C == K && (bits == 8 || bits == 4) && x_dt != XLA_AMD_DT_F32) {
+  if ((bits == 8 || bits == 4) && x_dt != XLA_AMD_DT_F32 && K % C == 0) {
     int per;
-    if (qmm_skinny_k_slices(M, N, K, bits, &per) > 1) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
+    if (qmm_skinny_k_slices(M, N, K, C, bits, &per) > 1) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
   }
   // many rows against blockwise or int4 weights: the tiled GEMM with per-block rounding points (the caller
   // must also have scale / zero point / result of x's dtype; else it takes the streaming kernel, pass by pass).

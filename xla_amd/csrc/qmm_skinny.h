@@ -14,13 +14,16 @@ struct SkinnyArgs {
   int scale_dt, zp_dt, out_dt;
   int dot_dt;    // dtype the dot product is rounded to before it is scaled (per-channel only)
   int store_dt;  // dtype of the stored tensor (out_dt, or a final cast of it)
-  // K slices over workgroups (per-channel weights only): blockIdx.y = slice of k_per_slice columns (a
+  // K slices over workgroups: blockIdx.y = slice of k_per_slice columns (a
   // multiple of the kernel's step, 512 columns for int8 and 1024 for int4; K when there is one slice).  With slices the kernel stores its raw sums instead
   // of results: part [slices][M][N] dot products, part_xs [slices][M] row sums of x (zero point only).
   int k_per_slice;
   int slices;
   float* part;
   float* part_xs;
+  // Blockwise weights (slices of whole quantization blocks): part holds the slices' sums of scale * round(block dot),
+  // part_z [slices][M][N] their sums of round(block sum of x) * zero point; both only need adding and the final roundings.
+  float* part_z;
 };
 
 int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);
@@ -29,4 +32,4 @@ int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t
 
 // K slices the streaming kernel should run a per-channel launch of M <= 32 rows in (1 = none):
 // few output channels against a long K, where every workgroup would otherwise copy all of x.
-int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int bits, int* k_per_slice);
+int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int64_t C, int bits, int* k_per_slice);

@@ -142,7 +142,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int ldk = a.K;
   const int k_begin = (int)blockIdx.y * a.k_per_slice;
   const int K = min(a.k_per_slice, ldk - k_begin);
-  const int N = a.N, M = a.M, C = a.slices > 1 ? K : a.C;
+  const int N = a.N, M = a.M, C = a.C == a.K ? K : a.C;  // per-channel: the slice is the one block
   const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
   const int x_dt = XT;
   const int scale_dt = UNI ? XT : a.scale_dt, zp_dt = UNI ? XT : a.zp_dt, out_dt = UNI ? XT : a.out_dt;
@@ -208,7 +208,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
   constexpr int kEntryBytes = 16 * RW * SE;          // one entry: the workgroup's channels
   constexpr int kSclTensor = kSclBytes / 2;          // the scales' entries, then the zero points'
   char* const xsm = smem + kSclBytes;
-  const int n_sblk = K / C;
+  const int n_sblk = ldk / a.C;       // quantization blocks of the whole K (blockwise)
+  const int sblk0 = k_begin / a.C;    // first block of this slice
   const int c_shift = (C & (C - 1)) == 0 ? __builtin_ctz(C) : -1;  // block size a power of two: shift instead of divide
   auto x_chunk_load = [&](int c) __attribute__((always_inline)) {
     const int c0 = c * CS;
@@ -227,7 +228,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
         const int ii = is_zp ? i - kInstr : i;
         const int e = ii * kEpi + lane / kPieces, piece = lane % kPieces;
         const int k_at = (c0 * SUB + e) * 128;
-        const int sblk = min(c_shift >= 0 ? (k_at >> c_shift) : k_at / C, n_sblk - 1);
+        const int sblk = min(sblk0 + (c_shift >= 0 ? (k_at >> c_shift) : k_at / C), n_sblk - 1);
         int ch = n_wg0 + piece * (4 / SE);
         if (ch + 4 / SE > N) ch = N - 4 / SE;    // channels past N: any valid address (never used)
         const char* src = (const char*)(is_zp ? a.zp : a.scale) + ((size_t)sblk * N + ch) * SE;
@@ -648,6 +649,17 @@ qmm_skinny_kernel(SkinnyArgs a) {
     const int n = n_wave + 4 * g;
     if (m < M && n < N) {
       constexpr float kBlockFactor = (RED != kRedRaw && BITS == 4 && kMfma) ? 16.0f : 1.0f;  // see block_epilogue
+      if constexpr (RED != kRedRaw) {
+        if (a.slices > 1) {
+          // one K slice of several (whole quantization blocks): the sums over this slice's blocks go to the workspace,
+          // a second kernel adds the slices and does the final roundings
+          const size_t at = ((size_t)blockIdx.y * M + m) * N + n;  // N % 4 == 0 for blockwise weights
+          *(f32x4*)(a.part + at) = f32x4{kBlockFactor * sacc[mt][0], kBlockFactor * sacc[mt][1], kBlockFactor * sacc[mt][2],
+                                         kBlockFactor * sacc[mt][3]};
+          if constexpr (HASZP) *(f32x4*)(a.part_z + at) = zacc[mt];
+          return;  // (this row tile is done)
+        }
+      }
       float o0 = qmm_round_dt(kBlockFactor * sacc[mt][0], out_dt), o1 = qmm_round_dt(kBlockFactor * sacc[mt][1], out_dt);
       float o2 = qmm_round_dt(kBlockFactor * sacc[mt][2], out_dt), o3 = qmm_round_dt(kBlockFactor * sacc[mt][3], out_dt);
       if constexpr (HASZP) {
@@ -817,7 +829,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
     a.N = (int)N; a.K = (int)K; a.C = (int)C;
     a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.out_dt = out_dt;
     a.dot_dt = dot_dt; a.store_dt = store_dt;
-    a.k_per_slice = (int)K; a.slices = 1; a.part = nullptr; a.part_xs = nullptr;
+    a.k_per_slice = (int)K; a.slices = 1; a.part = nullptr; a.part_xs = nullptr; a.part_z = nullptr;
     int rc;
     if (x_dt == XLA_AMD_DT_BF16) rc = qmm_skinny_launch_bf16(a, bits, zp != nullptr, (hipStream_t)stream);
     else if (x_dt == XLA_AMD_DT_F16) rc = qmm_skinny_launch_f16(a, bits, zp != nullptr, (hipStream_t)stream);

@@ -471,9 +471,49 @@ __global__ void __launch_bounds__(256) qmm_wo_gemm_finish_kernel(WoGemmArgs a, i
   else wo_store4<false>(a.out, m, n, a.N, o, dts.store_dt);
 }
 
+// The second kernel of K slices over blockwise weights: every slice left its sum over blocks of
+// scale * round(block dot) in part and of round(block sum of x) * zero point in part_z (or null);
+// out = round_out(sum), with a zero point round_out(out - round_zpo(sum of part_z)).
+// One thread per four consecutive channels of one row (N % 4 == 0).
+__global__ void __launch_bounds__(256) qmm_wo_bw_finish_kernel(const float* part, const float* part_z, void* out, int M,
+                                                               int N, int split, int out_dt, int zpo_dt, int store_dt) {
+  const int n4 = N / 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)M * n4) return;
+  const int m = (int)(idx / n4), n = (int)(idx % n4) * 4;
+  const size_t slice = (size_t)M * N, at = (size_t)m * N + n;
+  auto sum = [&](const float* p) {
+    f32x4 t = {0, 0, 0, 0};
+    int s = 0;
+    for (; s + 4 <= split; s += 4) {  // four loads in flight, additions in slice order
+      const f32x4 p0 = *(const f32x4*)(p + (size_t)s * slice), p1 = *(const f32x4*)(p + (size_t)(s + 1) * slice);
+      const f32x4 p2 = *(const f32x4*)(p + (size_t)(s + 2) * slice), p3 = *(const f32x4*)(p + (size_t)(s + 3) * slice);
+      t += p0; t += p1; t += p2; t += p3;
+    }
+    for (; s < split; ++s) t += *(const f32x4*)(p + (size_t)s * slice);
+    return t;
+  };
+  const f32x4 t = sum(part + at);
+  float o[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) o[v] = qmm_round_dt(t[v], out_dt);
+  if (part_z) {
+    const f32x4 z = sum(part_z + at);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) o[v] = qmm_round_dt(o[v] - qmm_round_dt(z[v], zpo_dt), out_dt);
+  }
+  wo_store4<true>(out, m, n, N, o, store_dt);
+}
+
 struct Plan {
   int mt, ng, split, k_per_split;
 };
+
+// floats of workspace for K slices of the weight-streaming kernel
+size_t slice_workspace_floats(int slices, int64_t M, int64_t N, bool blockwise) {
+  const size_t mn = (size_t)slices * (size_t)M * (size_t)N;
+  return blockwise ? 2 * mn : mn + (size_t)slices * (size_t)M;  // blockwise: room for the zero-point sums
+}
 
 // Tile and K split by shape.  Row tiles of 64 / 128 rows; 256 channels per workgroup
 // (128 when that is what fills the chip); K split over workgroups until about one workgroup
@@ -504,10 +544,11 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
 extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t C, int bits) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
   if (C <= 0) C = K;
-  if (C == K && M <= 32) {  // the weight-streaming kernel over K slices
+  if (K % C != 0) return 0;
+  if (M <= 32) {  // the weight-streaming kernel over K slices
     int per;
-    const int slices = qmm_skinny_k_slices(M, N, K, bits, &per);
-    if (slices > 1) return ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
+    const int slices = qmm_skinny_k_slices(M, N, K, C, bits, &per);
+    if (slices > 1) return slice_workspace_floats(slices, M, N, C != K) * sizeof(float);
   }
   if (C != K || bits != 8) return 0;  // blockwise / int4 weights: the tiled GEMM splits no K and needs no workspace
   size_t need = 0;
@@ -546,22 +587,35 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
   if (((uintptr_t)out & 15) && (N & 3) == 0)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: out must be 16-byte aligned");
   if (M == 0) return XLA_AMD_QMM_OK;
-  if (C == K && M <= 32) {
+  const bool blockwise = C != K;
+  // (blockwise weights in the weight-streaming kernel: every dtype but the stored one is x's, at least 8 scales)
+  const bool bw_ok = !blockwise || (scale_dt == x_dt && (!zp || zp_dt == x_dt) && dot_dt == x_dt && (K / C) * N >= 8 &&
+                                    (((uintptr_t)scale | (uintptr_t)zp) & 3) == 0);
+  if (M <= 32 && bw_ok) {
     // few rows: the weight-streaming kernel over K slices, when that is what its plan says and the workspace is there
     int per;
-    const int slices = qmm_skinny_k_slices(M, N, K, bits, &per);
-    const size_t need = ((size_t)slices * (size_t)M * (size_t)N + (size_t)slices * (size_t)M) * sizeof(float);
+    const int slices = qmm_skinny_k_slices(M, N, K, C, bits, &per);
+    const size_t need = slice_workspace_floats(slices, M, N, blockwise) * sizeof(float);
     if (slices > 1 && workspace && workspace_bytes >= need && (((uintptr_t)workspace) & 15) == 0) {
       SkinnyArgs k;
       k.x = x; k.w = (const uint8_t*)w_tiled; k.scale = scale; k.zp = zp; k.out = out;
-      k.M = (int)M; k.N = (int)N; k.K = (int)K; k.C = (int)K;
+      k.M = (int)M; k.N = (int)N; k.K = (int)K; k.C = (int)C;
       k.scale_dt = scale_dt; k.zp_dt = zp ? zp_dt : x_dt; k.out_dt = out_dt; k.dot_dt = dot_dt; k.store_dt = store_dt;
       k.k_per_slice = per; k.slices = slices;
       k.part = (float*)workspace;
-      k.part_xs = k.part + (size_t)slices * (size_t)M * (size_t)N;
+      const size_t mn = (size_t)slices * (size_t)M * (size_t)N;
+      k.part_xs = blockwise ? nullptr : k.part + mn;
+      k.part_z = blockwise && zp ? k.part + mn : nullptr;
       int rc = x_dt == XLA_AMD_DT_BF16 ? qmm_skinny_launch_bf16(k, bits, zp != nullptr, (hipStream_t)stream)
                                        : qmm_skinny_launch_f16(k, bits, zp != nullptr, (hipStream_t)stream);
       if (rc != XLA_AMD_QMM_OK) return rc;
+      if (blockwise) {
+        const int64_t threads = M * (N / 4);
+        hipLaunchKernelGGL(qmm_wo_bw_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                           (hipStream_t)stream, k.part, k.part_z, out, (int)M, (int)N, slices, out_dt,
+                           qmm_promote(x_dt, k.zp_dt), store_dt);
+        return QMM_CHECK_LAUNCH("weight_only_gemm blockwise finish launch");
+      }
       WoGemmArgs f;
       f.x = x; f.w = (const uint8_t*)w_tiled; f.scale = scale; f.zp = zp; f.out = out;
       f.part = k.part; f.part_xs = k.part_xs;
