@@ -168,6 +168,34 @@ def test_quantize_all_bf16_values(ops):
     assert torch.equal(s.cpu(), s_ref)
 
 
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+def test_quantize_every_pair_of_row_maximum_and_value(ops, xdt):
+  """Every positive finite value of the dtype as a row's maximum, against every value of the dtype no larger
+  than it: the whole domain of the quotient x / scale for 2-byte activations (the kernel divides by the row's
+  scale through a refined reciprocal and one correction step; this is the check that the result is the
+  division's, bit for bit).  The checker for all rows is the oracle's op sequence run by torch on the GPU
+  (a library division); every 499th row is also checked against the oracle on the CPU."""
+  bits = torch.arange(65536, dtype=torch.int32).to(torch.int16).cuda()
+  vals = bits.view(xdt)
+  vals = torch.where(torch.isfinite(vals.float()), vals, torch.zeros_like(vals))
+  maxima = vals[(vals.float() > 0)]
+  maxima = maxima[torch.argsort(maxima.float())]
+  assert maxima.numel() in (0x7f7f, 0x7bff)  # positive finite values, denormals included
+  chunk = 2048
+  for at in range(0, maxima.numel(), chunk):
+    mx = maxima[at:at + chunk].reshape(-1, 1)
+    x = torch.where(vals.float().abs().reshape(1, -1) <= mx.float(), vals.reshape(1, -1), torch.zeros((), dtype=xdt, device="cuda"))
+    for policy in ("wrap", "saturate"):  # (an f16 scale rounded in the subnormal range gives quotients up to 190)
+      q_ref, s_ref = oracle.quantize_tensor(x, overflow=policy)
+      q, s, _ = ops.quantize_per_token_gpu(x, overflow=policy)
+      bad = (q != q_ref).any(dim=1) | (s.view(torch.int16) != s_ref.view(torch.int16)).any(dim=1)
+      assert not bad.any(), f"{xdt} {policy}: rows with maximum {mx[bad][:4].flatten().tolist()} differ"
+    rows = torch.arange(at % 499, x.shape[0], 499)
+    if rows.numel():
+      q_cpu, s_cpu = oracle.quantize_tensor(x[rows.cuda()].cpu())
+      assert torch.equal(q[rows.cuda()].cpu(), q_cpu) and torch.equal(s[rows.cuda()].cpu(), s_cpu)
+
+
 # ---- W8A8: int32 accumulators bit exact, epilogue within tolerance ------------------------
 @pytest.mark.parametrize("m,n,k", [(64, 64, 64), (100, 130, 256), (256, 512, 128), (300, 700, 1024),
                                    (2048, 1024, 512), (7, 9, 80), (5, 8, 5), (512, 4096, 4096)])

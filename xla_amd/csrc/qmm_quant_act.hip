@@ -30,8 +30,39 @@ __device__ __forceinline__ int wave_sum(int v) {
   return v;
 }
 
-__device__ __forceinline__ int quantize_one(float xv, float scale, int x_dt, int policy) {
-  float r = rintf(qmm_round_dt(xv / scale, x_dt));  // rintf: round half to even
+// RN_f32(xv / scale) for a row's scale.  2-byte x with a scale well inside the f32 range: one
+// multiplication by the row's reciprocal (refined to within half an ulp once per row) and one
+// correction step on the exact remainder.  The result is then rounded to x's 8- or 11-bit
+// significand, which only asks for the f32 quotient to be exact where the true quotient is
+// representable (a tie of the narrower type is) and on the right side of every tie elsewhere:
+// the corrected quotient is within a fraction of an f32 ulp, x / scale of two such numbers
+// is never that close to a tie without being one.  (Checked against the division for every
+// pair of bf16 and of f16 values by the GPU tests.)  Otherwise: the IEEE division.
+struct RowDivisor {
+  float scale, rc;
+  bool fast;
+};
+template <int XT>
+__device__ __forceinline__ RowDivisor row_divisor(float scale) {
+  RowDivisor d;
+  d.scale = scale;
+  d.fast = XT != XLA_AMD_DT_F32 && scale > 1e-30f && scale < 1e30f;  // (false for NaN too)
+  float rc = __builtin_amdgcn_rcpf(scale);
+  rc = fmaf(fmaf(-scale, rc, 1.0f), rc, rc);
+  d.rc = rc;
+  return d;
+}
+__device__ __forceinline__ int quantize_one(float xv, const RowDivisor& d, int x_dt, int policy) {
+  if (d.fast) {
+    // Every x of the row is finite and at most 127.25 scales in magnitude (190.5 when an f16 scale was
+    // rounded in the subnormal range): no NaN, no infinity, nothing near the int32 range.
+    const float q0 = xv * d.rc;
+    const float q = fmaf(fmaf(-q0, d.scale, xv), d.rc, q0);
+    const float r = rintf(qmm_round_dt(q, x_dt));  // rintf: round half to even
+    if (policy == XLA_AMD_OVERFLOW_SATURATE) return (int)fminf(fmaxf(r, -128.f), 127.f);
+    return (int)(int8_t)(int)r;
+  }
+  float r = rintf(qmm_round_dt(xv / d.scale, x_dt));
   if (!(fabsf(r) <= 3.0e38f)) r = 0.f;              // NaN/inf (zero scale) -> 0
   if (policy == XLA_AMD_OVERFLOW_SATURATE) return (int)fminf(fmaxf(r, -128.f), 127.f);
   r = fminf(fmaxf(r, -2147483648.f), 2147483520.f);
@@ -108,6 +139,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
 #pragma unroll
   for (int i = 1; i < kThreads / 64; ++i) mx = nan_max(mx, smax[i]);
   const float scale = qmm_round_dt(mx / 127.0f, XT);
+  const RowDivisor divisor = row_divisor<XT>(scale);
 
   // pass 2: quantize
   int lsum = 0;
@@ -115,7 +147,7 @@ qmm_quantize_kernel(const void* __restrict__ x, int8_t* __restrict__ xq, void* _
     int q[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
-      q[i] = quantize_one(f[i], scale, XT, policy);
+      q[i] = quantize_one(f[i], divisor, XT, policy);
       lsum += q[i];
     }
     if constexpr (VEC == 1) {
