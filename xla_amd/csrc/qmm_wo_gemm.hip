@@ -69,12 +69,17 @@ constexpr int kLds = 160 * 1024;
 
 using namespace qmm_frag;
 
-template <int MT> struct WoCfg {
+template <int MT, int NG> struct WoCfg {
   static constexpr int BM = 16 * MT;
   static constexpr int X_TILE = BM * 256;                      // bytes of the x columns of one step (128 columns, 2-byte x)
-  static constexpr int kFit = kLds / (2 * X_TILE);             // steps per chunk slot that fit twice
+  // Weight blocks in flight per wave and channel group (register ring): two for the 64-row tile
+  // with two channel groups per wave, whose short steps (16 MFMAs per half block) would otherwise
+  // wait for memory every time and which has the registers; one for the others (four channel
+  // groups or 128 rows: the accumulators leave no room for a second block, and their steps are long).
+  static constexpr int P = (MT < 8 && NG == 2) ? 2 : 1;
+  static constexpr int kFit = kLds / (2 * X_TILE) / P * P;     // steps per chunk slot that fit twice (whole trips around the ring)
   static constexpr int CS = kFit < 8 ? kFit : 8;               // steps per chunk
-  static_assert(CS >= 1, "two chunk slots must fit in LDS");
+  static_assert(CS >= P, "two chunk slots must fit in LDS");
   static constexpr int lds_bytes(int steps) { return (steps <= CS ? steps : 2 * CS) * X_TILE; }
 };
 
@@ -157,7 +162,7 @@ struct WoItem {
 template <int XT, int MT, int NG, bool HASZP, bool UNI>
 __global__ void __launch_bounds__((kComputeWaves + kCopyWaves) * 64)
 qmm_wo_gemm_kernel(WoGemmArgs a) {
-  using Cfg = WoCfg<MT>;
+  using Cfg = WoCfg<MT, NG>;
   constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE, CS = Cfg::CS;
   constexpr int BN = 64 * NG;  // channels per workgroup: NG groups of 16 per computing wave
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -227,8 +232,9 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   // wave w owns the channel groups (n0/16 + w*NG) .. + NG-1 of the item's column tile
   const int n_blk = K / 128;  // blocks per channel group in the tiled weight
   const int groups = (N + 15) / 16;
+  constexpr int P = Cfg::P;
   const uint8_t* wp[NG];
-  i32x4 wreg[NG][2];
+  i32x4 wreg[P][NG][2];  // ring slot s % P holds the block of step s
   auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
@@ -236,18 +242,28 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * 2048 + lane * 16;
     });
   };
-  auto load_step = [&](int blk, auto hc) __attribute__((always_inline)) {
-    constexpr int h = hc;
+  auto load_half = [&](int blk, auto slotc, auto hc) __attribute__((always_inline)) {
+    constexpr int slot = slotc, h = hc;
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      wreg[gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * 2048 + h * 1024));
+      wreg[slot][gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * 2048 + h * 1024));
+    });
+  };
+  // the first P blocks of an item (a block past the end of a short item is the last one again: never used)
+  auto load_first = [&](const WoItem& w) __attribute__((always_inline)) {
+    qmm_static_for<P>([&](auto pc) {
+      constexpr int slot = pc;
+      const int blk = min(slot, w.steps - 1);
+      load_half(blk, qmm_const<slot>{}, qmm_const<0>{});
+      load_half(blk, qmm_const<slot>{}, qmm_const<1>{});
     });
   };
 
   f32x4 acc[NG][MT], xs[MT];
-  // one step (128 columns) out of LDS tile `tile`; the weight registers are refilled with
-  // block `next` as soon as each half has been used
-  auto compute = [&](int tile, int next, auto refillc) __attribute__((always_inline)) {
+  // one step (128 columns) out of LDS tile `tile` with the weights of ring slot SLOT; with
+  // REFILL the slot's registers are refilled with block `next` as soon as each half has been used
+  auto compute = [&](int tile, int next, auto slotc, auto refillc) __attribute__((always_inline)) {
+    constexpr int slot = slotc;
     constexpr bool kRefill = refillc != 0;
     const char* xbase = smem + tile * X_TILE;
     qmm_static_for<4>([&](auto jc) {
@@ -259,7 +275,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       });
       qmm_static_for<NG>([&](auto gc) {
         constexpr int gi = gc;
-        const i32x4 src = wreg[gi][j >> 1];
+        const i32x4 src = wreg[slot][gi][j >> 1];
         const i32x4 af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
         qmm_static_for<MT>([&](auto mc) {
           constexpr int mt = mc;
@@ -272,15 +288,23 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
           xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt], xs[mt]);
         });
       }
-      if constexpr (kRefill && (j & 1)) load_step(next, qmm_const<(j >> 1)>{});
+      if constexpr (kRefill && (j & 1)) load_half(next, qmm_const<slot>{}, qmm_const<(j >> 1)>{});
+    });
+  };
+  // P consecutive steps starting at step s (s % P == 0) of which `live` exist; NREF of them refill
+  // their slot (the refills are compile-time so that the loads in flight stay countable)
+  auto compute_group = [&](int tile, int s, int live, auto nrefc) __attribute__((always_inline)) {
+    constexpr int nref = nrefc;
+    qmm_static_for<P>([&](auto pc) {
+      constexpr int slot = pc;
+      if (slot == 0 || slot < live) compute(tile + slot, s + slot + P, qmm_const<slot>{}, qmm_const<(slot < nref ? 1 : 0)>{});
     });
   };
 
   int it = blockIdx.x;
   WoItem cur = item_of(it);
   set_weights(cur);
-  load_step(0, qmm_const<0>{});
-  load_step(0, qmm_const<1>{});
+  load_first(cur);
   int ring = 0;
   for (;;) {
     qmm_static_for<MT>([&](auto mc) {
@@ -292,10 +316,21 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     for (int c = 0; c < cur.n_chunks; ++c, ++ring) {
       qmm_bare_barrier();  // chunk `ring` is there (the copying waves waited for it)
       const int tile0 = (ring & 1) * CS - c * CS;
-      int s_end = min(cur.steps, (c + 1) * CS);
-      if (c + 1 == cur.n_chunks) --s_end;  // the item's last step fetches nothing more: it runs after the loop
-      for (; s < s_end; ++s) compute(tile0 + s, s + 1, qmm_const<1>{});
-      if (c + 1 == cur.n_chunks) compute(tile0 + s, 0, qmm_const<0>{});
+      if constexpr (P == 1) {
+        int s_end = min(cur.steps, (c + 1) * CS);
+        if (c + 1 == cur.n_chunks) --s_end;  // the item's last step fetches nothing more: it runs after the loop
+        for (; s < s_end; ++s) compute(tile0 + s, s + 1, qmm_const<0>{}, qmm_const<1>{});
+        if (c + 1 == cur.n_chunks) compute(tile0 + s, 0, qmm_const<0>{}, qmm_const<0>{});
+      } else {
+        const int s_end = min(cur.steps, (c + 1) * CS);
+        // groups of P steps (a chunk holds whole groups); the item's last P steps fetch nothing more
+        for (; s < s_end; s += P) {
+          const int left = cur.steps - s;
+          if (left >= 2 * P) compute_group(tile0 + s, s, P, qmm_const<P>{});
+          else if (left == 3) compute_group(tile0 + s, s, 2, qmm_const<1>{});
+          else compute_group(tile0 + s, s, left, qmm_const<0>{});
+        }
+      }
     }
 
     // the next item's first weights are requested before this item's results are stored: a wait
@@ -307,8 +342,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       it = it_next;
       cur = item_of(it);
       set_weights(cur);
-      load_step(0, qmm_const<0>{});
-      load_step(0, qmm_const<1>{});
+      load_first(cur);
     }
 
     // ---- results: four consecutive channels of one row per lane ----
@@ -392,7 +426,7 @@ int cu_count() {
 
 template <int XT, int MT, int NG>
 int launch(const WoGemmArgs& a, hipStream_t stream) {
-  using Cfg = WoCfg<MT>;
+  using Cfg = WoCfg<MT, NG>;
   const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + 64 * NG - 1) / (64 * NG)) * a.split;
   const int steps = a.k_per_split / 128;
   // one workgroup per compute unit (its LDS and registers leave room for no second one); each walks its share of the items
