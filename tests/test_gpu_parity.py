@@ -69,6 +69,21 @@ def test_skinny_per_channel_shapes(ops, m, n, k, xdt, zp):
   check(out, exp, "skinny per-channel")
 
 
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("zp", [False, True])
+def test_skinny_wide_outputs(ops, xdt, zp):
+  # more than 16384 channels: workgroups of eight computing waves (128 channels); one and two x tiles,
+  # a channel tail that ends inside a workgroup, inside a wave, and a whole number of workgroups
+  for (m, n, k) in [(16, 16400, 512), (32, 16500, 1024), (5, 20480, 640), (17, 16385, 128)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)
+    z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(xdt) if zp else None
+    exp = oracle.quantized_matmul(x, w, s, z)
+    before = ops.counters["skinny_mfma"]
+    out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z))
+    assert ops.counters["skinny_mfma"] == before + 1
+    check(out, exp, f"wide output {m, n, k, xdt, zp}")
+
+
 def test_per_channel_mixed_scale_dtype(ops):
   x, w, s, _ = cases.per_channel_int8(5, 64, 256, torch.bfloat16, torch.float32, seed=3)
   z = torch.randn(64, generator=cases.gen(6)) * 0.01

@@ -58,8 +58,9 @@ constexpr int kRedNone = 0;    // blockwise, KW == 1: nothing to reduce
 constexpr int kRedRaw = 1;     // per-channel (C == K, any KW): raw dot products and x sums are summed, then scaled
 constexpr int kRedScaled = 2;  // blockwise, KW > 1, whole blocks per step (KS % C == 0): scaled block results are summed
 
-// NW waves per workgroup; WSEG weight bytes per row per step.  Every launch uses the defaults
-// (4 waves, 512 bytes); an 8-wave shape with 256-byte steps measured slower and is not dispatched.
+// NW computing waves per workgroup; WSEG weight bytes per row per step.  Launches use 4 waves and
+// 512 bytes, or 8 waves for outputs of more than 16384 channels (see launch_split); an 8-wave
+// shape with 256-byte steps measured slower and is not dispatched.
 template <int XT, int BITS, int MT, int KW, int NW = kWaves, int WSEG = kWSeg>
 struct SkinnyCfg {
   static constexpr int RW = NW / KW;
@@ -746,6 +747,18 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
   if (can_split) {
     if (workgroups(2) <= kComputeUnits && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
     if (workgroups(4) <= kComputeUnits && steps >= 4 && SkinnyCfg<XT, BITS, MT, 4>::kFits) kw = 4;
+  }
+  // More than one round of 64-channel workgroups (N > 16384: the fused gate / up projection, a
+  // vocabulary projection): eight computing waves, 128 channels per workgroup.  Half as many
+  // copies of x out of L2 and no part-full second round; three waves per SIMD still fit the
+  // registers of the int8 per-channel kernels with one dtype throughout.  Measured with cold
+  // weights: 28672 x 4096 at M = 32 29.0 -> 25.9 us, at M = 16 24.8 -> 23.5; 18432 x 8192 at
+  // M = 1 37.4 -> 28.6 us (288 workgroups had been a round and an eighth).
+  if constexpr (BITS == 8 && XT != XLA_AMD_DT_F32) {
+    const bool uni = a.scale_dt == XT && a.zp_dt == XT && a.out_dt == XT && a.dot_dt == XT && a.store_dt == XT;
+    if (kw == 1 && perch && uni && workgroups(1) > kComputeUnits)
+      return haszp ? launch_kernel<XT, BITS, MT, 1, kRedRaw, true, true, 8, kWSeg>(a, stream)
+                   : launch_kernel<XT, BITS, MT, 1, kRedRaw, false, true, 8, kWSeg>(a, stream);
   }
   if (kw == 1) {
     return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
