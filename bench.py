@@ -194,6 +194,20 @@ def main():
                              "note": "one weight buffer, served from Infinity Cache; not HBM bandwidth"}
     del ws[1:]
 
+    # a launch long enough to amortise its fixed cost: the Llama-3 vocabulary projection (128256 x 4096, 525 MB) at M = 1;
+    # two weight copies in turn (1.05 GB: nothing of a copy is left in the 256 MB Infinity Cache when its turn comes)
+    gv = cases.gen(9)
+    wv = [torch.randint(-127, 128, (128256, K_IN), generator=gv, dtype=torch.int32).to(torch.int8).to(dev)]
+    wv.append(wv[0].clone())
+    sv = (torch.rand(128256, generator=gv) * 0.01).bfloat16().to(dev)
+    _, ev, _ = time_calls([(lambda w=w: op(xs[1], w, sv)) for w in wv], 24, 4, use_graph)
+    bv = gemv_bytes(1, 128256, K_IN)
+    extra["gemv_vocabulary_projection_128256x4096_M1_cold"] = {
+        "us": round(ev * 1e3, 2), "GBps": round(bv / ev / 1e6, 1), "frac_hbm": round(bv / ev / 1e6 / HBM_PEAK_GBPS, 4)}
+    for w in wv:
+      qmm.invalidate_weight_cache(w)  # frees the tiled copies too
+    del wv, sv, w
+
     # blockwise int4 (config 3)
     x3, w3, s3, z3, _ = cases.blockwise(16, 4096, 4096, 128, 4, torch.bfloat16, symmetric=False, seed=4)
     x3d, s3d, z3d = x3.to(dev), s3.to(dev), z3.to(dev)
