@@ -81,7 +81,8 @@ def test_dispatcher_regimes():
   tile = (ctypes.c_int32 * 3)()
   assert lib.xla_amd_qmm_w8a8_tile(2048, 14336, 4096, tile) == 0
   assert list(tile) == [256, 256, 128]
-  assert lib.xla_amd_qmm_w8a8_tile(64, 64, 64, tile) == 0 and list(tile)[:2] == [64, 32]  # few tiles: narrow ones
+  assert lib.xla_amd_qmm_w8a8_tile(64, 64, 64, tile) == 0 and list(tile)[:2] == [32, 32]  # few tiles: the smallest ones
+  assert lib.xla_amd_qmm_w8a8_tile(128, 4096, 4096, tile) == 0 and list(tile)[:2] == [64, 32]  # 512 tiles of 32 x 32 would be two per CU
   assert lib.xla_amd_qmm_w8a8_tile(32, 4096, 14336, tile) == 0 and list(tile)[:2] == [32, 32]
   assert lib.xla_amd_qmm_w8a8_tile(128, 14336, 4096, tile) == 0 and list(tile)[:2] == [64, 64]
   # the shape-based choice agrees with the measured best of the tuning sweep on the Llama-3-8B prefill shapes

@@ -75,28 +75,62 @@ def _add(batches, n_out, n_in, blocks):
       TUNED_BLOCK_SIZES[(_ARCH, bs, n_out, n_in, dtype, True)] = blocks
 
 
-# Fastest measured tile per shape (MI355X, one sweep over the four tile classes; ties
-# within 3 % go to what the library would pick by itself).  Shapes: the Llama-3-8B
-# linears (q/o, k/v, gate+up fused and single, qkv fused, down) and two square ones; launches of at most 128
-# 64 x 64 tiles take the 32-wide tiles measured afterwards (15-45 % faster there).
+# Fastest measured tile per shape (MI355X, one sweep over the six workgroup tiles, quantized Gaussian operands,
+# graph replays; a tile within 3 % of the fastest goes to what the library would pick by itself, which leaves four
+# entries that differ from the shape rule: (5120, 640) at 2048 / 4096 rows and (5120, 1280) at 2048 rows, where a
+# short K favours 128 x 128, and (37888, 3584) at 128 rows).  Shapes: the (out, in) pairs of the reference's table
+# (Llama-3-8B; Llama-3-70B, Qwen2.5-7B and a 5120-wide model sharded over devices) plus the single projections
+# and two square ones; batches as in the reference's table, 16 ... 16384 (where the result fits 700 M elements).
 # (n_out, n_in): {batch: (batch_block, out_block)}
 _MEASURED = {
-    (4096, 4096): {32: (32, 32), 64: (64, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64), 1024: (128, 128),
-                   2048: (128, 256), 4096: (256, 256), 8192: (256, 256)},
-    (1024, 4096): {32: (32, 32), 64: (64, 32), 128: (64, 32), 256: (64, 32), 512: (64, 32), 1024: (64, 64),
-                   2048: (64, 64), 4096: (64, 64), 8192: (128, 256)},
-    (14336, 4096): {32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (128, 128), 512: (128, 256), 1024: (256, 256),
-                    2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
-    (4096, 14336): {32: (32, 32), 64: (64, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64), 1024: (128, 128),
-                    2048: (128, 256), 4096: (256, 256), 8192: (256, 256)},
-    (6144, 4096): {32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64), 1024: (128, 256),
-                   2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
-    (28672, 4096): {32: (64, 64), 64: (64, 64), 128: (128, 128), 256: (128, 256), 512: (256, 256), 1024: (256, 256),
-                    2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
-    (8192, 8192): {32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128), 1024: (128, 256),
-                   2048: (256, 256), 4096: (256, 256), 8192: (256, 256)},
-    (2048, 2048): {32: (32, 32), 64: (64, 32), 128: (64, 32), 256: (64, 32), 512: (64, 64), 1024: (64, 64),
-                   2048: (64, 64), 4096: (128, 256), 8192: (256, 256)},
+    (6144, 4096): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (4096, 4096): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 128), 2048: (128, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (28672, 4096): {16: (64, 64), 32: (64, 64), 64: (64, 64), 128: (128, 128), 256: (128, 256), 512: (256, 256),
+                    1024: (256, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (4096, 14336): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64),
+                    1024: (128, 128), 2048: (128, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (1024, 4096): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (32, 32), 256: (32, 32), 512: (64, 32),
+                   1024: (64, 64), 2048: (64, 64), 4096: (128, 128), 8192: (128, 256), 16384: (256, 256)},
+    (14336, 4096): {16: (64, 64), 32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (128, 128), 512: (128, 256),
+                    1024: (256, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (8192, 8192): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (2048, 2048): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (32, 32), 256: (64, 32), 512: (64, 64),
+                   1024: (64, 64), 2048: (128, 128), 4096: (128, 256), 8192: (256, 256), 16384: (256, 256)},
+    (1280, 8192): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (32, 32), 256: (64, 32), 512: (64, 64),
+                   1024: (64, 64), 2048: (64, 64), 4096: (128, 256), 8192: (256, 256), 16384: (256, 256)},
+    (8192, 1024): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (7168, 8192): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (8192, 3584): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (4608, 3584): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (3584, 3584): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 128), 2048: (128, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (37888, 3584): {16: (64, 64), 32: (64, 64), 64: (64, 64), 128: (128, 128), 256: (256, 256), 512: (256, 256),
+                    1024: (256, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (3584, 18944): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (64, 32), 256: (64, 64), 512: (64, 64),
+                    1024: (128, 128), 2048: (128, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (896, 5120): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (32, 32), 256: (32, 32), 512: (64, 32),
+                  1024: (64, 64), 2048: (64, 64), 4096: (128, 128), 8192: (128, 256), 16384: (256, 256)},
+    (5120, 640): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64),
+                  1024: (128, 256), 2048: (128, 128), 4096: (128, 128), 8192: (256, 256), 16384: (256, 256)},
+    (5120, 1280): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 256), 2048: (128, 128), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (1792, 5120): {16: (32, 32), 32: (32, 32), 64: (32, 32), 128: (32, 32), 256: (64, 32), 512: (64, 64),
+                   1024: (64, 64), 2048: (128, 128), 4096: (128, 256), 8192: (256, 256), 16384: (256, 256)},
+    (13824, 5120): {16: (64, 64), 32: (64, 64), 64: (64, 64), 128: (64, 64), 256: (128, 128), 512: (128, 256),
+                    1024: (256, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (5120, 6912): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (6912, 5120): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (128, 128),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
+    (5120, 3456): {16: (32, 32), 32: (32, 32), 64: (64, 32), 128: (64, 64), 256: (64, 64), 512: (64, 64),
+                   1024: (128, 256), 2048: (256, 256), 4096: (256, 256), 8192: (256, 256), 16384: (256, 256)},
 }
 for (_n_out, _n_in), _by_batch in _MEASURED.items():
   for _bs, (_bm, _bn) in _by_batch.items():
