@@ -48,12 +48,6 @@ extern "C" size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits) {
   return bits == 8 ? rows * (size_t)K : rows * (size_t)K / 2;
 }
 
-// The two regimes of a quantized linear layer on MI355X:
-//  * few rows of x (decode): every weight byte is used M times, far below the
-//    ~630 int8 ops/byte (or ~310 bf16 flops/byte) the chip can do per HBM
-//    byte, so the weight is streamed exactly once by the skinny kernel;
-//  * many rows with int8 activations (prefill): LDS-tiled int8 MFMA GEMM.
-// Shapes neither fast kernel accepts run the one-thread-per-output kernels.
 // K slices over workgroups for the weight-streaming kernel.  A workgroup of that kernel owns 64
 // (or 32, 16) output channels over all of K and copies every column of x it multiplies; with few
 // channels and a long K the workgroups together copy several times the weight's bytes of x (out
@@ -87,9 +81,14 @@ int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int64_t C, int bits, in
   return (int)slices;
 }
 
+// The two regimes of a quantized linear layer on MI355X:
+//  * few rows of x (decode): every weight byte is used M times, far below the
+//    ~630 int8 ops/byte (or ~310 bf16 flops/byte) the chip can do per HBM
+//    byte, so the weight is streamed exactly once by the skinny kernel;
+//  * many rows with int8 activations (prefill): LDS-tiled int8 MFMA GEMM.
+// Shapes neither fast kernel accepts run the one-thread-per-output kernels.
 extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, int bits,
                                     int x_dt, int quantize_activation) {
-  (void)N;
   if (quantize_activation) {
     if (K % 64 == 0 && M * N >= 64 * 64) return XLA_AMD_KERNEL_W8A8_MFMA;
     return XLA_AMD_KERNEL_W8A8_GENERIC;
@@ -98,6 +97,7 @@ extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, 
   // many rows of 2-byte x against per-channel int8 weights: the tiled GEMM reads the weight once
   // per 128 rows, the streaming kernel once per 32
   if (C == K && bits == 8 && K % 128 == 0 && x_dt != XLA_AMD_DT_F32 && M > 32) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
+  // few rows against few channels and a long K: the streaming kernel over K slices, behind the GEMM's entry point
   if ((bits == 8 || bits == 4) && x_dt != XLA_AMD_DT_F32 && K % C == 0) {
     int per;
     if (qmm_skinny_k_slices(M, N, K, C, bits, &per) > 1) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
