@@ -7,14 +7,17 @@ with every input already resident in HBM.  The weight rotates over enough
 distinct copies (> 512 MB) that neither L2 nor the 256 MB Infinity Cache can
 hold it, so the reported bandwidth is HBM bandwidth.  The K timed steps are
 captured once into a HIP graph and replayed (a decode step is launch-bound
-otherwise); `--no-graph` times eager calls instead.
+otherwise); `--no-graph` times eager calls instead.  Before every timed
+replay the graph is replayed untimed for PREWARM_MS, so that the chip is at
+the clocks it sustains under the workload, not in the low power state the
+host-side set-up leaves it in.
 
 Prints ONE JSON line.  `value` is algorithmic GB/s of the whole timed region
 (wall clock between device synchronisations); `roofline` is the same kernel
 measured with HIP events on its stream; `cpu_baseline` is the CPU oracle timed
 on this host; `extra` carries the other configurations (M=1/4, hot cache,
-blockwise int4, W8A8 prefill GEMM with its own MFMA roofline, the 7 linears of
-a Llama-3-8B layer).
+a vocabulary projection, blockwise int4, W8A8 prefill GEMM with its own MFMA
+roofline, the weight-only prefill GEMMs, the 7 linears of a Llama-3-8B layer).
 """
 import argparse
 import json
