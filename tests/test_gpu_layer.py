@@ -267,6 +267,51 @@ def test_graph_capture_needs_a_prepared_weight(ops):
     check(op(xd, wd, sd), exp, "eager between replays")
 
 
+def test_graph_replays_of_the_routes_with_several_kernels(ops):
+  """One HIP graph over the routes that launch more than one kernel or use a workspace (K slices of per-channel and of
+  blockwise weights with their second kernel, the weight-only GEMM with a K split, the W8A8 operator's quantizer + GEMM):
+  every replay, with new activations copied in and eager work in between, gives the eager result."""
+  op = torch.ops.xla.quantized_matmul
+  m = 24
+  x1, w1, s1, _ = cases.per_channel_int8(m, 512, 8192, torch.bfloat16, torch.bfloat16, seed=61)      # K slices
+  x2, w2, s2, z2, _ = cases.blockwise(m, 256, 8192, 128, 4, torch.bfloat16, symmetric=False, seed=62)  # blockwise K slices
+  x3, w3, s3, _ = cases.per_channel_int8(80, 384, 2048, torch.bfloat16, torch.bfloat16, seed=63)     # tiled GEMM, K split
+  x4 = cases.outlier_activations(96, 1024, torch.bfloat16, seed=64)                                  # W8A8
+  _, w4, s4, _ = cases.per_channel_int8(1, 320, 1024, torch.bfloat16, torch.float32, seed=65)
+  dev_ = lambda *ts: [t.cuda() for t in ts]
+  x1d, w1d, s1d = dev_(x1, w1, s1)
+  x2d, w2d, s2d, z2d = dev_(x2, w2, s2, z2)
+  x3d, w3d, s3d = dev_(x3, w3, s3)
+  x4d, w4d, s4d = dev_(x4, w4, s4)
+  ops.prepare_weight(w1d)
+  ops.prepare_weight(w2d, block_size=128, int4_weight=True)
+  ops.prepare_weight(w3d)
+
+  def run():
+    return (op(x1d, w1d, s1d), op(x2d, w2d, s2d, z2d, 128, True), op(x3d, w3d, s3d),
+            op(x4d, w4d, s4d, quantize_activation=True))
+
+  before = ops.counters["wo_gemm"]
+  run()
+  assert ops.counters["wo_gemm"] == before + 3
+  torch.cuda.synchronize()
+  g = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(g):
+    outs = run()
+  gen = cases.gen(66)
+  for rep in range(3):
+    for xd in (x1d, x2d, x3d, x4d):  # new activations for this replay
+      xd.copy_((torch.randn(xd.shape, generator=gen) * (1 + rep)).to(xd.dtype))
+    g.replay()
+    torch.cuda.synchronize()
+    eager = run()
+    torch.cuda.synchronize()
+    for i, (a, b) in enumerate(zip(outs, eager)):
+      assert torch.equal(a, b), f"replay {rep}, route {i}"
+  check(outs[0], oracle.quantized_matmul(x1d.cpu(), w1, s1), "K slices after the replays")
+  check(outs[1], oracle.quantized_matmul(x2d.cpu(), w2, s2, z2, block_size=128, int4_weight=True), "blockwise K slices after the replays")
+
+
 def test_quantizer_nan_row(ops):
   x = cases.outlier_activations(6, 512, torch.bfloat16, seed=2)
   x[2, 100] = float("nan")
