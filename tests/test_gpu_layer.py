@@ -54,8 +54,9 @@ def test_config5_decode_m32(ops, layer, name):
   x = torch.randn(32, k, generator=cases.gen(7)).bfloat16()
   s16 = s.bfloat16()
   exp = oracle.quantized_matmul(x, w, s16)
-  # the down projection (few channels, long K) runs the streaming kernel over K slices, through the workspace entry point
-  which = "wo_gemm" if name == "down" else "skinny_mfma"
+  # the down projection (few channels, long K) and the narrow k / v projections (two x tiles) run the streaming kernel
+  # over K slices, through the workspace entry point
+  which = "wo_gemm" if name in ("down", "k", "v") else "skinny_mfma"
   before = ops.counters[which]
   out = torch.ops.xla.quantized_matmul(x.cuda(), w.cuda(), s16.cuda())
   assert ops.counters[which] == before + 1

@@ -58,7 +58,9 @@ def test_wo_gemm_shapes(ops, xdt, zp):
                     # more work items than compute units: workgroups walk several of them
                     (60, 33024, 256),
                     # few rows against a long K: the weight-streaming kernel over K slices (N tail, M tail, 28 and 16 steps)
-                    (32, 200, 8192), (9, 4096, 14336), (24, 1000, 8192)]:
+                    (32, 200, 8192), (9, 4096, 14336), (24, 1000, 8192),
+                    # a narrow output with two x tiles: K slices at K = 4096 too
+                    (32, 1024, 4096), (17, 520, 4096)]:
     x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)
     z = (torch.randn(n, generator=cases.gen(5)) * 0.01).to(xdt) if zp else None
     exp = oracle.quantized_matmul(x, w, s, z)

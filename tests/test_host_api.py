@@ -73,6 +73,8 @@ def test_dispatcher_regimes():
   assert d(32, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(4, 4096, 14336, 14336, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # too few rows of x to matter
   assert d(32, 4096, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA       # K too short for slices
+  assert d(32, 1024, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # ... unless the output is narrow and x two tiles high
+  assert d(16, 1024, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA
   assert d(32, 14336, 8192, 8192, 8, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA      # enough workgroups already
   assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(32, 4096, 14336, 14336, 8) == 4 * (32 * 4096 + 32) * 4  # four K slices
   assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(2048, 14336, 4096, 4096, 8) == 0

@@ -65,10 +65,12 @@ int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int64_t C, int bits, in
     else if (ks % C != 0) return 1;
   }
   if (M > 32 || K % ks != 0) return 1;
-  // (measured with cold weights at M = 32: 4096 x 14336 25.5 -> 17.8 us; with K = 4096 or fewer than 8 rows the
-  // second kernel costs more than the copies saved)
-  if (M < 8 || K < 8192) return 1;
+  // (measured with cold weights at M = 32: 4096 x 14336 25.5 -> 17.8 us; with fewer than 8 rows the second kernel
+  // costs more than the copies saved, and so it does with K = 4096 unless the output is narrow and x two tiles
+  // high: 1024 x 4096 at M = 32 8.6 -> 7.5 us, 2048 x 4096 8.8 -> 8.4, but 4096 x 4096 9.4 -> 9.9)
   const int64_t cols = (N + 63) / 64;
+  if (M < 8 || K < 4096) return 1;
+  if (K < 8192 && !(M > 16 && cols <= 16)) return 1;
   if (cols >= 128) return 1;  // enough workgroups of 64 channels already
   const int64_t steps = K / ks;
   int64_t slices = 256 / cols;
