@@ -44,6 +44,85 @@ def gemv_bytes(m, n, k, w_bytes_per_elem=1.0, x_b=2, s_b=2, out_b=2, n_scale_row
   return int(n * k * w_bytes_per_elem + m * k * x_b + scale_bytes + m * n * out_b)
 
 
+def timeline(torch, _lib, qmm, cases, dev, m, hot):
+  """In-kernel timeline of the decode GEMV (x bf16 [m,4096], w int8 [14336,4096]).
+
+  The diagnostic build of the streaming kernel notes, per wave, the chip-wide 100 MHz
+  counter at fixed points (entry, first weights requested / landed, first x chunk in
+  LDS, every step, exit) and the shader clock counter at entry and exit.  The launch
+  that is read back is the last node of a HIP graph of launches over rotating weight
+  copies (cold weights, as in the benchmark), replayed until the clocks have settled.
+  """
+  import ctypes
+  import numpy as np
+  lib = _lib.load()
+  raw = ctypes.CDLL(_lib.lib_path())
+  raw.xla_amd_qmm_timeline_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+  raw.xla_amd_qmm_timeline_read.restype = ctypes.c_int
+  x, w_cpu, s_cpu, _ = cases.per_channel_int8(m, N_OUT, K_IN, torch.bfloat16, torch.bfloat16, seed=2)
+  x, s_d, w0 = x.to(dev), s_cpu.to(dev), w_cpu.to(dev)
+  wt0 = qmm._tiled_weight(w0, 8, _lib.W_NK)
+  n_rot = 1 if hot else 12
+  wts = [wt0] + [wt0.clone() for _ in range(n_rot - 1)]
+  out = torch.empty(m, N_OUT, dtype=torch.bfloat16, device=dev)
+  bf = _lib.DT_BF16
+
+  def run(wt):
+    _lib.check(lib.xla_amd_qmm_weight_only_skinny(x.data_ptr(), wt.data_ptr(), s_d.data_ptr(), None, out.data_ptr(), m,
+                                                  N_OUT, K_IN, K_IN, 8, bf, bf, bf, bf, bf, bf,
+                                                  torch.cuda.current_stream().cuda_stream), "weight_only_skinny")
+
+  for wt in wts:
+    run(wt)
+  torch.cuda.synchronize()
+  g = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(g):
+    for i in range(24):
+      run(wts[i % n_rot])
+  t_pre = time.perf_counter()
+  while (time.perf_counter() - t_pre) * 1e3 < PREWARM_MS:
+    g.replay()
+    torch.cuda.synchronize()
+  n_blocks, n_waves, n_notes = 2048, 12, 32
+  host = np.zeros(n_blocks * n_waves * n_notes, dtype=np.uint64)
+  rc = raw.xla_amd_qmm_timeline_read(host.ctypes.data_as(ctypes.c_void_p), host.size)
+  assert rc == 0, "timeline_read failed"
+  t = host.reshape(n_blocks, n_waves, n_notes).astype(np.int64)
+  live = t[:, :, 0] > 0
+  nb, nwv = int(live.any(axis=1).sum()), int(live[0].sum())
+  ncomp = nwv - 4  # the last four waves of a workgroup copy x
+  t0 = t[:, :, 0][live].min()
+  rel = np.where(t > 0, (t - t0) * 0.01, np.nan)  # 100 MHz ticks -> us since the first wave's entry
+  print(f"decode GEMV x bf16 [{m},{K_IN}] x w int8 [{N_OUT},{K_IN}], {'one weight copy (cache-resident)' if hot else '12 rotating weight copies (cold)'}: "
+        f"{nb} workgroups x ({ncomp} computing + {nwv - ncomp} copying waves)")
+
+  def table(title, waves, names):
+    print(f"{title}: min / median / max over waves, us since the first wave's entry")
+    for i, name in names:
+      v = rel[:nb, waves, i].ravel()
+      v = v[~np.isnan(v)]
+      if v.size:
+        print(f"  {name:34s} {v.min():7.2f} {np.median(v):7.2f} {v.max():7.2f}")
+
+  n_steps = K_IN // 512
+  table("computing waves", slice(0, ncomp),
+        [(0, "entry"), (1, "first weights requested"), (2, "first weights landed"), (3, "first x chunk in LDS (met)")] +
+        [(4 + i, f"step {i} done") for i in range(min(n_steps - 1, 22))] +
+        [(28, "all steps done"), (29, "k-split sums in LDS"), (30, "results stored, leaves")])
+  table("copying waves", slice(ncomp, nwv),
+        [(0, "entry"), (1, "first chunk requested"), (2, "first chunk landed"), (3, "first meeting passed")] +
+        [(4 + i, f"chunk {i + 1} landed") for i in range(8)] + [(30, "leaves")])
+  end = np.nanmax(rel[:nb, :nwv, 30], axis=1)
+  print(f"first entry to last exit: {end.max():.2f} us; exit of a workgroup's last wave: min {end.min():.2f}, "
+        f"median {np.median(end):.2f}, max {end.max():.2f}")
+  steps = rel[:nb, :ncomp, 4:4 + min(n_steps - 1, 22)]
+  d = np.diff(steps, axis=2).reshape(-1, steps.shape[2] - 1)
+  print("duration of steps 1.., median over waves (us):", " ".join(f"{v:.2f}" for v in np.nanmedian(d, axis=0)))
+  clk = (t[:nb, :ncomp, 27] - t[:nb, :ncomp, 26]).astype(np.float64)
+  dur = (t[:nb, :ncomp, 30] - t[:nb, :ncomp, 0]).astype(np.float64) * 0.01
+  print(f"shader clock over the computing waves' lifetime: median {np.median(clk / dur):.0f} MHz")
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -52,6 +131,11 @@ def main():
   ap.add_argument("--no-graph", action="store_true", help="time eager calls instead of a HIP graph replay")
   ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--timeline", action="store_true",
+                  help="instead of the benchmark: in-kernel timeline of the decode GEMV (diagnostic build of the "
+                       "streaming kernel, libxla_amd_qmm_timeline.so); prints a table, not the JSON line")
+  ap.add_argument("--timeline-hot", action="store_true", help="with --timeline: one weight copy (cache-resident) instead of rotating ones")
+  ap.add_argument("--timeline-m", type=int, default=16, help="with --timeline: rows of x")
   ap.add_argument("--calibrate-copy", action="store_true",
                   help="also run a plain 256 MiB device copy (known traffic, for scaling rocprof byte counters)")
   args = ap.parse_args()
@@ -65,6 +149,9 @@ def main():
     print("bench.py: no GPU visible", file=sys.stderr)
     sys.exit(3)
   from xla_amd import _lib
+  if args.timeline:
+    # the diagnostic build of the library takes the place of the regular one for this process
+    _lib._LIB_PATH = os.path.join(os.path.dirname(_lib._LIB_PATH), "libxla_amd_qmm_timeline.so")
   _lib.load()  # no fallback: fail here if the HIP library is missing
   import xla_amd.experimental.custom_kernel  # noqa: F401
   import xla_amd.experimental.xla_quantized_matmul as qmm
@@ -150,6 +237,10 @@ def main():
     return found[0] if found else None
 
   use_graph = not args.no_graph
+
+  if args.timeline:
+    timeline(torch, _lib, qmm, cases, dev, args.timeline_m, args.timeline_hot)
+    return
 
   if args.calibrate_copy:
     src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)

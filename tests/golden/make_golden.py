@@ -93,6 +93,40 @@ def main():
     rows.append(dict(values=vals, word=word))
   out["int4_pack"] = rows
 
+  # 7. the five bf16 rounding points of the blockwise path with a zero point
+  #    (xla_quantized_matmul.py:119-133: p = einsum('scn,...sc->...sn'), out = einsum('sn,...sn->...n'),
+  #    zsum = x.sum(-1), zpo = zsum @ zp, out - zpo; every result is a bf16 tensor).  Inputs are chosen so
+  #    that every sum is exact in f32 whatever the order (x multiples of 1/16, |w| <= 8), hence the only
+  #    inexact operations are the five roundings, done here with the exact model's round_to_format.
+  def blockwise_bf16_case(m, s_, c, n, tag):
+    xq = rng.integers(-255, 256, size=(m, s_ * c)) / 16.0                    # bf16-exact (8 significant bits)
+    wq4 = rng.integers(-8, 8, size=(s_, c, n))
+    sc_ = bf16_grid((1.0 + rng.integers(0, 128, size=(s_, n)) / 128.0) * 2.0 ** rng.integers(-9, -5, size=(s_, n)))
+    zp_ = bf16_grid(rng.integers(-8, 8, size=(s_, n)) * sc_)
+    xr_ = xq.reshape(m, s_, c)
+
+    def run(r_p=True, r_o1=True, r_zs=True, r_zpo=True, r_o2=True):
+      rnd = lambda v, on: bf16_grid(v) if on else v
+      p_ = rnd(np.einsum("scn,msc->msn", wq4.astype(np.float64), xr_), r_p)
+      o_ = rnd(np.einsum("sn,msn->mn", sc_, p_), r_o1)
+      zs = rnd(xr_.sum(-1), r_zs)
+      zo = rnd(zs @ zp_, r_zpo)
+      return rnd(o_ - zo, r_o2), rnd(o_, True)
+
+    full, no_zp = run()
+    # a formulation that skips any one of the five roundings must fail this fixture
+    for k in range(5):
+      flags = [True] * 5
+      flags[k] = False
+      other, _ = run(*flags)
+      assert (other != full).any(), f"{tag}: rounding point {k} does not show in this fixture"
+    out[tag] = dict(m=m, s=s_, c=c, n=n, x_bits=bx.f64_to_bf16_bits(xq).tolist(), w=wq4.tolist(),
+                    scale_bits=bx.f64_to_bf16_bits(sc_).tolist(), zp_bits=bx.f64_to_bf16_bits(zp_).tolist(),
+                    expect_bits=bx.f64_to_bf16_bits(no_zp).tolist(), expect_zp_bits=bx.f64_to_bf16_bits(full).tolist())
+
+  blockwise_bf16_case(2, 3, 4, 4, "blockwise_bf16_roundings")          # any kernel that takes odd shapes
+  blockwise_bf16_case(3, 3, 128, 8, "blockwise_bf16_roundings_c128")   # a shape the streaming kernel takes
+
   with open(os.path.join(HERE, "quantized_matmul_golden.json"), "w") as f:
     json.dump(out, f)
   print("wrote", os.path.join(HERE, "quantized_matmul_golden.json"), "overflow band counts", counts)

@@ -363,6 +363,27 @@ def test_golden_overflow_band_and_w8a8(ops):
   assert torch.equal(acc.cpu().long(), torch.tensor(g["acc"]))
 
 
+@pytest.mark.parametrize("tag", ["blockwise_bf16_roundings", "blockwise_bf16_roundings_c128"])
+def test_golden_blockwise_bf16_rounding_points(ops, tag):
+  """The five bf16 rounding points of the blockwise path, fixed by the exact model (every sum of the fixture is
+  exact in f32, so the kernels' summation order cannot show): generic kernel (C = 4), streaming kernel (C = 128,
+  int8 container and packed int4), bit for bit."""
+  g = GOLD[tag]
+  m, s_, c, n = g["m"], g["s"], g["c"], g["n"]
+  x = _bf16_from_bits(np.asarray(g["x_bits"])).reshape(m, s_ * c).contiguous()
+  w = torch.tensor(g["w"], dtype=torch.int8)
+  scale = _bf16_from_bits(np.asarray(g["scale_bits"])).reshape(s_, n).contiguous()
+  zp = _bf16_from_bits(np.asarray(g["zp_bits"])).reshape(s_, n).contiguous()
+  expect = _bf16_from_bits(np.asarray(g["expect_bits"])).reshape(m, n)
+  expect_zp = _bf16_from_bits(np.asarray(g["expect_zp_bits"])).reshape(m, n)
+  before = dict(ops.counters)
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, scale), block_size=c).cpu(), expect)
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, scale, zp), block_size=c).cpu(), expect_zp)
+  assert torch.equal(torch.ops.xla.quantized_matmul(*dev(x, w, scale, zp), block_size=c, int4_weight=True).cpu(), expect_zp)
+  kernel = "skinny_mfma" if c % 128 == 0 else "generic"
+  assert ops.counters[kernel] == before[kernel] + 3, "the fixture did not reach the kernel it is meant for"
+
+
 def test_golden_dot_general_and_int4_pack(ops):
   from xla_amd import _lib
   g = GOLD["dot_general_int32"]

@@ -67,6 +67,30 @@ def test_dot_general_int32_exact():
     assert torch.equal(got.long(), torch.tensor(g["expect"][i]))
 
 
+def _blockwise_bf16_fixture(tag):
+  g = GOLD[tag]
+  m, s_, c, n = g["m"], g["s"], g["c"], g["n"]
+  x = bf16_from_bits(np.asarray(g["x_bits"])).reshape(m, s_ * c)
+  w = torch.tensor(g["w"], dtype=torch.int8)
+  scale, zp = bf16_from_bits(np.asarray(g["scale_bits"])).reshape(s_, n), bf16_from_bits(np.asarray(g["zp_bits"])).reshape(s_, n)
+  return x, w, scale, zp, c, bf16_from_bits(np.asarray(g["expect_bits"])).reshape(m, n), bf16_from_bits(
+      np.asarray(g["expect_zp_bits"])).reshape(m, n)
+
+
+@pytest.mark.parametrize("tag", ["blockwise_bf16_roundings", "blockwise_bf16_roundings_c128"])
+def test_blockwise_bf16_rounding_points(tag):
+  """The five points where the blockwise path rounds to bf16 (every sum of the fixture is exact in f32,
+  so the roundings are the only inexact operations; the generator checks that dropping any one of them
+  changes the result): oracle and the operator's CPU formulation, bit for bit."""
+  import xla_amd.experimental.xla_quantized_matmul  # noqa: F401  (registers the CPU key)
+  x, w, scale, zp, c, expect, expect_zp = _blockwise_bf16_fixture(tag)
+  assert torch.equal(oracle.quantized_matmul(x, w, scale, block_size=c), expect)
+  assert torch.equal(oracle.quantized_matmul(x, w, scale, zp, block_size=c), expect_zp)
+  assert torch.equal(torch.ops.xla.quantized_matmul(x, w, scale, block_size=c), expect)
+  assert torch.equal(torch.ops.xla.quantized_matmul(x, w, scale, zp, block_size=c), expect_zp)
+  assert torch.equal(torch.ops.xla.quantized_matmul(x, w, scale, zp, block_size=c, int4_weight=True), expect_zp)
+
+
 # ---- quantizer against the independent exact model ---------------------------------
 @pytest.mark.parametrize("policy", ["saturate", "wrap"])
 def test_quantizer_all_bf16_values(policy):

@@ -39,6 +39,13 @@ SOURCES = [
     ("qmm_linear.hip", [], "qmm_linear.o"),
 ]
 
+# Diagnostic library: the same objects with the bf16 unit of the streaming kernel compiled with
+# -DQMM_SKINNY_TIMELINE (every wave records when it reaches fixed points of the kernel; read back by
+# `python bench.py --timeline`).  Never loaded by the operators.
+TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libxla_amd_qmm_timeline.so")
+TIMELINE_UNIT = ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=1", "-DQMM_SKINNY_TIMELINE"], "qmm_skinny_bf16_timeline.o")
+TIMELINE_REPLACES = "qmm_skinny_bf16.o"
+
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # packed-fp32 instructions are switched off on purpose (hipcc otherwise forms
@@ -104,12 +111,13 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     return obj, kernels
 
   with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-    results = list(ex.map(compile_one, SOURCES))
+    results = list(ex.map(compile_one, SOURCES + [TIMELINE_UNIT]))
+  timeline_obj, timeline_kernels = results.pop()
   objs = [r[0] for r in results]
   kernels = [k for r in results for k in r[1]]
   with open(RESOURCES_PATH, "w") as f:
     json.dump(kernels, f, indent=1)
-  spilling = [k for k in kernels if k.get("scratch_bytes_per_lane", 0) > 0]
+  spilling = [k for k in kernels + timeline_kernels if k.get("scratch_bytes_per_lane", 0) > 0]
   if spilling:
     raise RuntimeError("kernels with a scratch frame (register spills):\n" +
                        "\n".join("  %s: %s (%d bytes per lane, %d VGPRs)" % (k["unit"], k["kernel"], k["scratch_bytes_per_lane"],
@@ -117,6 +125,10 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
   tmp = LIB_PATH + ".tmp"
   _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] + objs)
   os.replace(tmp, LIB_PATH)
+  tmp = TIMELINE_LIB_PATH + ".tmp"
+  _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] +
+       [timeline_obj if os.path.basename(o) == TIMELINE_REPLACES else o for o in objs])
+  os.replace(tmp, TIMELINE_LIB_PATH)
   return LIB_PATH
 
 

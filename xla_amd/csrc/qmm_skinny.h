@@ -24,6 +24,8 @@ struct SkinnyArgs {
   // Blockwise weights (slices of whole quantization blocks): part holds the slices' sums of scale * round(block dot),
   // part_z [slices][M][N] their sums of round(block sum of x) * zero point; both only need adding and the final roundings.
   float* part_z;
+  // Diagnostic build of the kernel only (its time notes): offset of their LDS area, -1 = none.
+  int tl_off = -1;
 };
 
 int qmm_skinny_launch_f32(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream);

@@ -45,6 +45,39 @@
 #include "qmm_frag.h"
 #include "qmm_skinny.h"
 
+// Diagnostic build (-DQMM_SKINNY_TIMELINE, a library of its own; see xla_amd/build.py): every wave
+// notes the time (the chip-wide 100 MHz counter) at fixed points of the kernel - entry, first
+// weights requested / landed, first x chunk there, each step, end - in LDS and writes its notes
+// to qmm_tl_buf when it leaves; xla_amd_qmm_timeline_read copies them to the host.  The regular
+// build compiles none of it.
+#ifdef QMM_SKINNY_TIMELINE
+constexpr int kTlSlots = 32;        // notes per wave
+constexpr int kTlWaves = 12;        // waves per workgroup at most
+constexpr int kTlBlocks = 2048;     // workgroups per launch at most (larger launches are not recorded)
+constexpr int kTlLdsBytes = kTlWaves * kTlSlots * 8;
+__device__ uint64_t qmm_tl_buf[kTlBlocks * kTlWaves * kTlSlots];
+// (no branch around a note: every lane stores the same value to the same LDS address; a branch
+// inside the main loop would make the compiler's wait counts for the weight ring conservative)
+// (explicit LDS pointers: a generic pointer would make these flat stores, which count as global
+// memory operations too and turn every wait of the ring into a wait for all loads)
+typedef volatile __attribute__((address_space(3))) uint64_t* qmm_tl_ptr_t;
+#define QMM_TL_AREA ((qmm_tl_ptr_t)(__attribute__((address_space(3))) char*)smem + a.tl_off / 8)
+#define QMM_TL(i) \
+  do { QMM_TL_AREA[wave * kTlSlots + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define QMM_TL_CLK(i) do { QMM_TL_AREA[wave * kTlSlots + (i)] = __builtin_readcyclecounter(); } while (0)
+#define QMM_TL_DUMP()                                                                                    \
+  do {                                                                                                   \
+    QMM_TL_CLK(27);                                                                                      \
+    if (lane < kTlSlots)                                                                                 \
+      qmm_tl_buf[((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * kTlWaves + wave) * kTlSlots + lane] =  \
+          QMM_TL_AREA[wave * kTlSlots + lane];                                                           \
+  } while (0)
+#else
+#define QMM_TL(i) do {} while (0)
+#define QMM_TL_CLK(i) do {} while (0)
+#define QMM_TL_DUMP() do {} while (0)
+#endif
+
 namespace {
 
 using namespace qmm_frag;
@@ -139,6 +172,11 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int rw = wave % RW, kw = wave / RW;
   const int r = lane & 15, g = lane >> 4;
+#ifdef QMM_SKINNY_TIMELINE
+  if (lane < kTlSlots) QMM_TL_AREA[wave * kTlSlots + lane] = 0;
+#endif
+  QMM_TL(0);  // entry
+  QMM_TL_CLK(26);
   // this workgroup's K slice: columns k_begin .. k_begin + K of rows that hold ldk columns
   const int ldk = a.K;
   const int k_begin = (int)blockIdx.y * a.k_per_slice;
@@ -281,7 +319,9 @@ qmm_skinny_kernel(SkinnyArgs a) {
     // previous launch having pushed the code out of L2)
     if (__builtin_expect(wave >= NW, 0)) {
       x_chunk_load(0);
+      QMM_TL(1);  // first copies requested
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's copies have landed
+      QMM_TL(2);  // ... landed
       for (int c = 0; c < n_chunks; ++c) {
         if (kSlots == 1 && c > 0) {
           qmm_bare_barrier();  // every wave has finished reading the old columns
@@ -289,12 +329,16 @@ qmm_skinny_kernel(SkinnyArgs a) {
           __builtin_amdgcn_s_waitcnt(0x0F70);
         }
         qmm_bare_barrier();    // chunk c is there (and, with two slots, chunk c - 1 has been read)
+        if (c == 0) QMM_TL(3);
         if (kSlots == 2 && c + 1 < n_chunks) {
           x_chunk_load(c + 1);
           __builtin_amdgcn_s_waitcnt(0x0F70);
+          QMM_TL(4 + min(c, 21));  // chunk c + 1 landed
         }
       }
       if constexpr (KW > 1) { qmm_bare_barrier(); qmm_bare_barrier(); }  // the two of the k-split reduction
+      QMM_TL(30);
+      QMM_TL_DUMP();
       return;
     }
   }
@@ -303,6 +347,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // before anything else is computed.
   qmm_static_for<P>([&](auto pc) { load_regs(pc, pc); });
   __builtin_amdgcn_sched_barrier(0);
+  QMM_TL(1);  // first weights requested
   if constexpr (kCopiers == 0) {
     // Loads complete in order, so waiting for the copies also waits for those weights, which
     // step 0 needs anyway.
@@ -537,7 +582,9 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // First chunk: weights of step 0 are under way (issued at the top of the kernel) and so
   // are the x copies (with the blockwise scales of their sub-steps).
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the first weights (and this wave's copies, if it copies) have landed
+  QMM_TL(2);  // first weights landed
   qmm_bare_barrier();
+  QMM_TL(3);  // first x chunk there
   fetch_channel_scales();  // (per-channel) needed at the very end: their latency hides behind the main loop
   int s0 = 0;  // this wave's next step
   for (int c = 0; c < n_chunks; ++c) {
@@ -567,12 +614,14 @@ qmm_skinny_kernel(SkinnyArgs a) {
         // (a step past the end, which only occurs to complete a trip around the
         // ring, has every sub-step beyond K: it issues its loads and computes nothing)
         compute(hc, tile0 + min(gs - c0, nst - 1), s, qmm_const<1>{});
+        QMM_TL(4 + min(s, 21));  // this wave's step s done
       });
     }
     if constexpr (KW == 1 && P == 1) {
       if (c + 1 == n_chunks) compute(qmm_const<0>{}, tile0 + s0 - c0, s0, qmm_const<0>{});
     }
   }
+  QMM_TL(28);  // all steps done
 
   // ---- reduction over k-splits, final rounding, store ------------------------------------
   const int zpo_dt = qmm_promote(x_dt, zp_dt);
@@ -595,7 +644,12 @@ qmm_skinny_kernel(SkinnyArgs a) {
       if constexpr (RED == kRedRaw && NEEDXS) mine[(4 * MT + mt) * 64] = xs[mt][0];
     });
     __syncthreads();
-    if (kw != 0) return;
+    if (kw != 0) {
+      QMM_TL(30);
+      QMM_TL_DUMP();
+      return;
+    }
+    QMM_TL(29);  // partial sums of the k-splits are in LDS
     qmm_static_for<MT>([&](auto mc) {
       constexpr int mt = mc;
       qmm_static_for<4>([&](auto vc) {
@@ -639,6 +693,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
           }
         }
       });
+      QMM_TL(30);
+      QMM_TL_DUMP();
       return;
     }
     block_epilogue(0, qmm_const<0>{});  // the single block ends here
@@ -691,6 +747,8 @@ qmm_skinny_kernel(SkinnyArgs a) {
       }
     }
   });
+  QMM_TL(30);  // results stored (requested)
+  QMM_TL_DUMP();
 }
 
 template <int XT, int BITS, int MT, int KW, int RED, bool HASZP, bool UNI, int NW = kWaves, int WSEG = kWSeg>
@@ -702,13 +760,27 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
     auto kern = qmm_skinny_kernel<XT, BITS, MT, KW, RED, HASZP, UNI, NW, WSEG>;
     static std::atomic<uint64_t> lds_set{0};
     constexpr int kSlots = skinny_slots<Cfg, MT, RED, KW>();
-    const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20, kSlots) + skinny_scale_bytes<Cfg, XT, MT, RED, KW>(), lds_set, "weight_only_skinny hipFuncSetAttribute");
+#ifdef QMM_SKINNY_TIMELINE
+    constexpr int kMaxLds = 160 * 1024;  // (room for the time notes wherever the kernel leaves it)
+#else
+    constexpr int kMaxLds = Cfg::lds_bytes(1 << 20, kSlots) + skinny_scale_bytes<Cfg, XT, MT, RED, KW>();
+#endif
+    const int rc = qmm_set_max_lds((const void*)kern, kMaxLds, lds_set, "weight_only_skinny hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
     const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
     const int steps = (a.k_per_slice + Cfg::KS - 1) / Cfg::KS;
     constexpr int kScl = skinny_scale_bytes<Cfg, XT, MT, RED, KW>();
-    hipLaunchKernelGGL(kern, dim3(blocks, (unsigned)a.slices), dim3((NW + skinny_copier_waves<MT, RED>()) * 64),
-                       Cfg::lds_bytes(steps, kSlots) + kScl, stream, a);
+    int lds = Cfg::lds_bytes(steps, kSlots) + kScl;
+#ifdef QMM_SKINNY_TIMELINE
+    SkinnyArgs at = a;
+    if (lds + kTlLdsBytes > 160 * 1024 || (uint64_t)blocks * a.slices > kTlBlocks)
+      return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_skinny (timeline build): no room for the time notes of this launch");
+    at.tl_off = lds;
+    lds += kTlLdsBytes;
+    hipLaunchKernelGGL(kern, dim3(blocks, (unsigned)a.slices), dim3((NW + skinny_copier_waves<MT, RED>()) * 64), lds, stream, at);
+#else
+    hipLaunchKernelGGL(kern, dim3(blocks, (unsigned)a.slices), dim3((NW + skinny_copier_waves<MT, RED>()) * 64), lds, stream, a);
+#endif
     return QMM_CHECK_LAUNCH("weight_only_skinny launch");
   }
 }
@@ -797,6 +869,14 @@ int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t
 int qmm_skinny_launch_bf16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t stream) {
   return launch_bits<XLA_AMD_DT_BF16>(a, bits, haszp, stream);
 }
+
+#ifdef QMM_SKINNY_TIMELINE
+// The notes of the last recorded launch: [workgroup][wave (12)][note (32)] of 100 MHz ticks, 0 = not reached.
+extern "C" int xla_amd_qmm_timeline_read(uint64_t* host, size_t count) {
+  if (!host || count > sizeof(qmm_tl_buf) / sizeof(uint64_t)) return qmm_fail(XLA_AMD_QMM_EINVAL, "timeline_read: bad arguments");
+  return qmm_check_hip(hipMemcpyFromSymbol(host, HIP_SYMBOL(qmm_tl_buf), count * sizeof(uint64_t)), "timeline_read");
+}
+#endif
 
 extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled, const void* scale,
                                               const void* zp, void* out, int64_t M, int64_t N,

@@ -149,7 +149,9 @@ def _relayout(w: torch.Tensor, bits: int, layout: int, kind: str) -> torch.Tenso
   if nbytes == 0:
     raise RuntimeError(f"xla_amd: cannot re-lay out weight of shape {tuple(w.shape)} to {bits} bits ({kind})")
   out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
-  _lib.check(copy_fn(w.data_ptr(), out.data_ptr(), s, c, n, layout, bits, _lib.stream_of(w)), f"{kind} weight")
+  # (the copy is keyed on the caller's tensor; a strided weight is read through a contiguous temporary, once)
+  src = w if w.is_contiguous() else w.contiguous()
+  _lib.check(copy_fn(src.data_ptr(), out.data_ptr(), s, c, n, layout, bits, _lib.stream_of(w)), f"{kind} weight")
   counters["pack"] += 1
   if hit is None:
     weakref.finalize(w, _pack_cache.pop, key, None)
@@ -195,7 +197,7 @@ def prepare_weight(w: torch.Tensor, block_size: int = -1, int4_weight: bool = Fa
   bits = 4 if int4_weight else 8
   if _lib.load().xla_amd_qmm_dispatch(1, n, k, c, bits, _lib.dt(x_dtype), 0) != _lib.KERNEL_SKINNY_MFMA:
     return False
-  _tiled_weight(w.contiguous() if not w.is_contiguous() else w, bits, layout)
+  _tiled_weight(w, bits, layout)
   return True
 
 
@@ -245,6 +247,7 @@ def _weight_only_launch(x2, w, w_tiled, n, k, c, layout, bits, scaler, zero_poin
     if w is None:
       raise RuntimeError("xla_amd: this shape runs the generic kernel, which reads the operator's weight layout")
     counters["generic"] += 1
+    w = w.contiguous()
     _lib.check(
         lib.xla_amd_qmm_weight_only_generic(x2.data_ptr(), w.data_ptr(), scaler.data_ptr(),
                                             _lib.ptr(zero_point), out.data_ptr(), m, n, k, c, layout,
@@ -309,12 +312,11 @@ def quantized_matmul_gpu(x, w, scaler, zero_point=None, block_size=-1, int4_weig
     raise RuntimeError(f"xla_amd quantized_matmul: x and scaler must be floating point, got {x.dtype}, {scaler.dtype}")
   out_dtype = _result_dtype(x, scaler, quantize_activation)
   x2 = x.reshape(-1, x.shape[-1]).contiguous()
-  w = w.contiguous()
   scaler = scaler.contiguous()
   if zero_point is not None:
     zero_point = zero_point.contiguous()
   if quantize_activation:
-    out = w8a8_linear_gpu(x2, w, scaler, zero_point, x_scale_dtype=x2.dtype, cvt_dtype=scaler.dtype,
+    out = w8a8_linear_gpu(x2, w.contiguous(), scaler, zero_point, x_scale_dtype=x2.dtype, cvt_dtype=scaler.dtype,
                           mid_dtype=scaler.dtype, out_dtype=out_dtype)
     if store_dtype is not None and store_dtype != out_dtype:
       out = out.to(store_dtype)
@@ -567,7 +569,7 @@ class XlaQuantizedLinear(torch.nn.Module):
     if _lib.load().xla_amd_qmm_dispatch(1, n, k, c, bits, _lib.DT_BF16, 0) != _lib.KERNEL_SKINNY_MFMA:
       return False
     invalidate_weight_cache(w)
-    self._weight_tiled = _tiled_weight(w.contiguous(), bits, layout)
+    self._weight_tiled = _tiled_weight(w, bits, layout)
     self._tiled_from = (_version_of(w), w.data_ptr())
     if release_weight:
       invalidate_weight_cache(w)  # the module's own reference keeps the copy alive
@@ -593,14 +595,32 @@ class XlaQuantizedLinear(torch.nn.Module):
       state_dict[prefix + "weight"] = module._rebuilt_weight()
     return state_dict
 
-  def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+  def _restore_weight(self):
+    """Brings the operator-layout `weight` back from the tiled form (undoes `release_weight`)."""
     if self._released_shape is not None:
-      self.weight = torch.empty(self._released_shape, dtype=torch.int8, device=self.weight.device)
-      self._weight_tiled = None
+      self.weight = self._rebuilt_weight()
       self._released_shape = None
-    else:
+      self._weight_tiled = None
+
+  def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+    # A dict without this layer's `weight` (a partial or scaler-only checkpoint, strict=False) leaves the
+    # weight as it is, tiled copy included.  A dict with one is copied into a buffer that already holds the
+    # current values (rebuilt from the tiled form when that was all the module kept), so that a load which
+    # fails half-way - a shape mismatch is only reported, not copied - still leaves a valid weight.
+    if prefix + "weight" in state_dict:
+      self._restore_weight()
       self._weight_tiled = None
     return super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+  def _apply(self, fn, recurse=True):
+    # .cpu() / .to(other device) of a module that kept only the tiled form: the operator layout can only be
+    # rebuilt where the tiled copy lives, so it is rebuilt before the move (and the module needs a new
+    # prepare() afterwards).  Casts and moves that stay on the device keep the released state.
+    if self._released_shape is not None:
+      here = self._weight_tiled.device
+      if fn(torch.empty(0, dtype=torch.uint8, device=here)).device != here:
+        self._restore_weight()
+    return super()._apply(fn, recurse)
 
   def _tiled_is_current(self):
     if self._weight_tiled is None:
