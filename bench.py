@@ -123,6 +123,52 @@ def timeline(torch, _lib, qmm, cases, dev, m, hot):
   print(f"shader clock over the computing waves' lifetime: median {np.median(clk / dur):.0f} MHz")
 
 
+def stream_probe(torch, _lib, dev):
+  """Kernels that only read the decode GEMV's weight bytes (14336 x 4096 = 58.7 MB), shaped like its memory side:
+  `grid` workgroups of `waves` waves, each wave keeping `depth` 1 KB loads in flight over its own region.
+  Per-launch time as a node of a HIP graph over 12 rotating buffers (cold) and over one buffer (cache-resident)."""
+  import ctypes
+  raw = ctypes.CDLL(_lib.lib_path())
+  fn = raw.xla_amd_qmm_diag_stream
+  fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p] + [ctypes.c_int] * 4 + [ctypes.c_void_p]
+  fn.restype = ctypes.c_int
+  total = N_OUT * K_IN
+  bufs = [torch.ones(total + (1 << 20), dtype=torch.uint8, device=dev) for _ in range(12)]
+  sink = torch.zeros(4, dtype=torch.int32, device=dev)
+  print(f"streaming {total / 1e6:.1f} MB: us per launch (graph node), cold = 12 rotating buffers, hot = one buffer")
+  print(f"{'grid':>5} {'waves':>5} {'KB in flight/wave':>18} {'cold us':>8} {'TB/s':>5} {'hot us':>7}")
+  for grid, waves, depth in [(224, 4, 8), (256, 4, 8), (256, 4, 4), (256, 4, 16), (256, 8, 4), (256, 8, 8), (512, 4, 8),
+                             (1024, 4, 8)]:
+    kb = -(-total // 1024 // (grid * waves))
+    times = []
+    for hot in (False, True):
+      def launch(b):
+        rc = fn(b.data_ptr(), sink.data_ptr(), grid, waves, depth, kb, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+      for b in bufs:
+        launch(b)
+      torch.cuda.synchronize()
+      g = torch.cuda.CUDAGraph()
+      with torch.cuda.graph(g):
+        for i in range(48):
+          launch(bufs[0 if hot else i % 12])
+      t_pre = time.perf_counter()
+      while (time.perf_counter() - t_pre) * 1e3 < PREWARM_MS:
+        g.replay()
+        torch.cuda.synchronize()
+      best = 1e9
+      for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(5):
+          g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) * 1e3 / (5 * 48))
+      times.append(best)
+    print(f"{grid:5d} {waves:5d} {depth:18d} {times[0]:8.2f} {total / times[0] / 1e6:5.2f} {times[1]:7.2f}")
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -134,6 +180,9 @@ def main():
   ap.add_argument("--timeline", action="store_true",
                   help="instead of the benchmark: in-kernel timeline of the decode GEMV (diagnostic build of the "
                        "streaming kernel, libxla_amd_qmm_timeline.so); prints a table, not the JSON line")
+  ap.add_argument("--stream-probe", action="store_true",
+                  help="instead of the benchmark: time kernels that only read the decode GEMV's 58.7 MB, for several "
+                       "launch shapes (diagnostic library); prints a table")
   ap.add_argument("--timeline-hot", action="store_true", help="with --timeline: one weight copy (cache-resident) instead of rotating ones")
   ap.add_argument("--timeline-m", type=int, default=16, help="with --timeline: rows of x")
   ap.add_argument("--calibrate-copy", action="store_true",
@@ -149,7 +198,7 @@ def main():
     print("bench.py: no GPU visible", file=sys.stderr)
     sys.exit(3)
   from xla_amd import _lib
-  if args.timeline:
+  if args.timeline or args.stream_probe:
     # the diagnostic build of the library takes the place of the regular one for this process
     _lib._LIB_PATH = os.path.join(os.path.dirname(_lib._LIB_PATH), "libxla_amd_qmm_timeline.so")
   _lib.load()  # no fallback: fail here if the HIP library is missing
@@ -240,6 +289,9 @@ def main():
 
   if args.timeline:
     timeline(torch, _lib, qmm, cases, dev, args.timeline_m, args.timeline_hot)
+    return
+  if args.stream_probe:
+    stream_probe(torch, _lib, dev)
     return
 
   if args.calibrate_copy:

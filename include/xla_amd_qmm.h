@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define XLA_AMD_QMM_ABI_VERSION 3
+#define XLA_AMD_QMM_ABI_VERSION 4
 
 /* return codes */
 #define XLA_AMD_QMM_OK 0
@@ -95,26 +95,40 @@ int xla_amd_qmm_pack_weight(const int8_t* w, void* packed, int64_t S, int64_t C,
                             int src_layout, int bits, void* stream);
 
 /*
- * Bytes of the tiled copy of a weight that the streaming kernel reads:
- * ceil(N/16)*16 * K for bits == 8, half of that for bits == 4.  Needs
- * K % 128 == 0; returns 0 for arguments the tile kernel rejects.
+ * Channels per group of the tiled copy of a weight [N, K] with quantization
+ * blocks of C columns (C == K or C <= 0: per-channel): 16, except that
+ * per-channel int8 weights of 4096 channels or more are tiled in groups of
+ * 14, 12 or 10 channels when that fills the chip's 1024 wave slots better
+ * (14336 channels: groups of 14, 1024 waves instead of 896).  Host.
  */
-size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits);
+int xla_amd_qmm_tile_group(int64_t N, int64_t K, int64_t C, int bits);
+
+/*
+ * Bytes of the tiled copy of a weight that the streaming kernel reads:
+ * ceil(N/G)*G * K for bits == 8 (G = xla_amd_qmm_tile_group), half of that
+ * for bits == 4.  Needs K % 128 == 0; returns 0 for arguments the tile kernel
+ * rejects.
+ */
+size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int64_t C, int bits);
 
 /*
  * One-time re-layout of a weight into the tiled form the streaming kernel
  * reads (same arguments and the same reference statement as
  * xla_amd_qmm_pack_weight: values are unchanged, only storage).  Needs
- * K % 128 == 0.  For every group g of 16 consecutive channels and every
- * sub-step t of 128 consecutive columns there is one block of BLK bytes at
- * byte offset (g * (K/128) + t) * BLK; channels past N are stored as zero.
- *   bits 8 (BLK 2048): byte h*1024 + l*16 + j (h in 0..1, l in 0..63, j in 0..15)
- *           holds w(16g + l%16, 128t + 32*(l/16) + 16h + j).
- *   bits 4 (BLK 1024): the 32-bit word at byte l*16 + 4i (i in 0..3) holds the
- *           8 columns 128t + 32*(l/16) + 8i .. +7 of channel 16g + l%16 in the
+ * K % 128 == 0.  With G = xla_amd_qmm_tile_group(N, K, C, bits) there is, for
+ * every group p of G consecutive channels and every sub-step t of 128
+ * consecutive columns, one block of BLK bytes at byte offset
+ * (p * (K/128) + t) * BLK; channels past N are stored as zero.
+ *   bits 8 (BLK 128 G): byte ((h*4 + q)*G + r)*16 + j (h in 0..1, q in 0..3, r in 0..G-1,
+ *           j in 0..15) holds w(G p + r, 128t + 32q + 16h + j).
+ *   bits 4 (BLK 1024, G = 16): the 32-bit word at byte (q*16 + r)*16 + 4i (i in 0..3) holds the
+ *           8 columns 128t + 32q + 8i .. +7 of channel 16p + r in the
  *           nibble order of xla_amd_qmm_pack_weight.
- * A 64-lane load of 16 bytes per lane from consecutive addresses thus puts
- * into lane l exactly the MFMA operand fragment of channel l%16.
+ * With G = 16 a 64-lane load of 16 bytes per lane from consecutive addresses
+ * puts into lane l = 16q + r exactly the MFMA operand fragment of channel r;
+ * with a narrower group lane 16q + r' reads row r' - (G p % 4) of quarter q
+ * (clamped to 0..G-1), so that the lane's four results are the channels
+ * 4 floor(G p / 4) + 4q .. +3: four-aligned, as with groups of 16.
  */
 int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, int64_t N,
                             int src_layout, int bits, void* stream);

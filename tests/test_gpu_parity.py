@@ -400,6 +400,35 @@ def test_golden_dot_general_and_int4_pack(ops):
     assert packed.tolist() == [r["word"] for r in rows]
 
 
+def _tiled_expected(wn, bits, G):
+  """The tiled copy by its written definition (include/xla_amd_qmm.h): groups of G channels."""
+  n, k = wn.shape
+  groups, n_blk = (n + G - 1) // G, k // 128
+  blk = 128 * G if bits == 8 else 64 * G
+  expect = np.zeros(groups * n_blk * blk, dtype=np.uint8)
+  P = [0, 2, 4, 6, 1, 3, 5, 7]
+  for p in range(groups):
+    for t in range(n_blk):
+      base = (p * n_blk + t) * blk
+      for q in range(4):
+        for r in range(G):
+          ch, k0 = G * p + r, 128 * t + 32 * q
+          if ch >= n:
+            continue
+          if bits == 8:
+            for h in range(2):
+              at = base + ((h * 4 + q) * G + r) * 16
+              expect[at:at + 16] = wn[ch, k0 + 16 * h:k0 + 16 * h + 16] & 0xFF
+          else:
+            for i in range(4):
+              word = 0
+              for j in range(8):
+                word |= ((int(wn[ch, k0 + 8 * i + P[j]]) + 8) & 15) << (4 * j)
+              for b in range(4):
+                expect[base + (q * G + r) * 16 + 4 * i + b] = (word >> (8 * b)) & 0xFF
+  return expect
+
+
 def test_tile_weight_layout(ops):
   # the tiled copy against its written definition (include/xla_amd_qmm.h), both source layouts, N tail
   from xla_amd import _lib
@@ -408,32 +437,44 @@ def test_tile_weight_layout(ops):
   for bits in (8, 4):
     lo, hi = (-128, 128) if bits == 8 else (-8, 8)
     w = torch.randint(lo, hi, (n, k), generator=g, dtype=torch.int32).to(torch.int8)
-    wn = w.numpy().astype(np.int64)
-    groups, n_blk = (n + 15) // 16, k // 128
-    blk = 2048 if bits == 8 else 1024
-    expect = np.zeros(groups * n_blk * blk, dtype=np.uint8)
-    P = [0, 2, 4, 6, 1, 3, 5, 7]
-    for gi in range(groups):
-      for t in range(n_blk):
-        base = (gi * n_blk + t) * blk
-        for l in range(64):
-          ch, k0 = 16 * gi + l % 16, 128 * t + 32 * (l // 16)
-          if ch >= n:
-            continue
-          if bits == 8:
-            for h in range(2):
-              for j in range(16):
-                expect[base + h * 1024 + l * 16 + j] = wn[ch, k0 + 16 * h + j] & 0xFF
-          else:
-            for i in range(4):
-              word = 0
-              for j in range(8):
-                word |= ((int(wn[ch, k0 + 8 * i + P[j]]) + 8) & 15) << (4 * j)
-              for b in range(4):
-                expect[base + l * 16 + 4 * i + b] = (word >> (8 * b)) & 0xFF
+    expect = _tiled_expected(w.numpy().astype(np.int64), bits, 16)
     for layout, src in ((_lib.W_NK, w), (_lib.W_SCN, w.T.reshape(2, 128, n).contiguous())):
       got = ops._tiled_weight(src.cuda(), bits, layout).cpu().numpy()
-      assert got.shape == expect.shape and np.array_equal(got, expect), (bits, layout)
+      assert got.shape == expect.shape and (got == expect).all(), f"bits {bits} layout {layout}"
+
+
+@pytest.mark.parametrize("n,group", [(4100, 10), (6144, 12), (7165, 14), (7166, 14)])
+def test_tile_weight_layout_narrow_groups(ops, n, group):
+  # per-channel int8 weights of many channels are tiled in groups of 14 / 12 / 10 channels: layout by its
+  # definition, and the way back to the operator's layout
+  from xla_amd import _lib
+  lib = _lib.load()
+  k = 256
+  assert lib.xla_amd_qmm_tile_group(n, k, k, 8) == group
+  w = torch.randint(-128, 128, (n, k), generator=cases.gen(11), dtype=torch.int32).to(torch.int8)
+  expect = _tiled_expected(w.numpy().astype(np.int64), 8, group)
+  tiled = ops._tiled_weight(w.cuda(), 8, _lib.W_NK)
+  got = tiled.cpu().numpy()
+  assert got.shape == expect.shape and (got == expect).all()
+  back = torch.empty_like(w, device="cuda")
+  _lib.check(lib.xla_amd_qmm_untile_weight(tiled.data_ptr(), back.data_ptr(), 1, k, n, _lib.W_NK, 8, _lib.stream_of(back)),
+             "untile_weight")
+  assert torch.equal(back.cpu(), w)
+
+
+@pytest.mark.parametrize("n", [4100, 6144, 7165, 7166, 14336])
+@pytest.mark.parametrize("m", [1, 16, 32, 80, 200])
+@pytest.mark.parametrize("zp", [False, True])
+def test_narrow_channel_groups_parity(ops, n, m, zp):
+  """Per-channel int8 weights whose tiled copy has groups of 10 / 12 / 14 / 14 / 14 channels: the streaming
+  kernel (m <= 32) and the tiled GEMM (more rows) against the oracle; 4100, 7166 and 7165 channels also take
+  the stores of rows that are not a multiple of four (of two) channels long."""
+  k = 512
+  x, w, s, _ = cases.per_channel_int8(m, n, k, torch.bfloat16, torch.bfloat16, seed=n + m)
+  z = (torch.randn(n, generator=cases.gen(3)) * 0.01).to(torch.bfloat16) if zp else None
+  expected = oracle.quantized_matmul(x, w, s, z)
+  got = torch.ops.xla.quantized_matmul(*dev(x, w, s, z))
+  check(got, expected, f"n={n} m={m} zp={zp}")
 
 
 def test_w8a8_tiles_and_tails(ops):

@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
   for n in names:
     assert hasattr(lib, n), f"{n} declared in the header but not exported"
   assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-  assert lib.xla_amd_qmm_abi_version() == 3
+  assert lib.xla_amd_qmm_abi_version() == 4
 
 
 def test_header_cites_reference_for_each_entry_point():
@@ -102,9 +102,18 @@ def test_error_codes_without_gpu():
   assert lib.xla_amd_qmm_packed_bytes(8, 64, 8) == 512
   assert lib.xla_amd_qmm_packed_bytes(8, 64, 4) == 256
   assert lib.xla_amd_qmm_packed_bytes(8, 5, 4) == 0
-  assert lib.xla_amd_qmm_tiled_bytes(17, 256, 8) == 32 * 256
-  assert lib.xla_amd_qmm_tiled_bytes(16, 128, 4) == 16 * 64
-  assert lib.xla_amd_qmm_tiled_bytes(16, 64, 8) == 0
+  assert lib.xla_amd_qmm_tiled_bytes(17, 256, 256, 8) == 32 * 256
+  assert lib.xla_amd_qmm_tiled_bytes(16, 128, 128, 4) == 16 * 64
+  assert lib.xla_amd_qmm_tiled_bytes(16, 64, 64, 8) == 0
+  # channel groups of the tiled copy: 16, narrower where that fills the 1024 wave slots of the chip better
+  # (per-channel int8 weights of 4096 channels or more only)
+  group = lib.xla_amd_qmm_tile_group
+  assert [group(n, 4096, 4096, 8) for n in (1024, 4096, 5120, 6144, 8192, 11008, 14336, 16384, 28672, 128256)] == \
+      [16, 16, 10, 12, 16, 12, 14, 16, 14, 16]
+  assert group(14336, 4096, 4096, 4) == 16 and group(14336, 4096, 128, 8) == 16 and group(14336, 4096, -1, 8) == 14
+  assert lib.xla_amd_qmm_tiled_bytes(14336, 4096, 4096, 8) == 14336 * 4096          # 1024 groups of 14
+  assert lib.xla_amd_qmm_tiled_bytes(7165, 256, 256, 8) == 512 * 14 * 256            # groups of 14, three channels of padding
+  assert lib.xla_amd_qmm_tiled_bytes(7165, 256, 128, 8) == 448 * 16 * 256            # blockwise: groups of 16
   rc = lib.xla_amd_qmm_weight_only_skinny(None, None, None, None, None, 1, 1, 128, 128, 8, 1, 1, 1, 1, 1, 1, None)
   assert rc == _lib.EINVAL and b"null" in lib.xla_amd_qmm_last_error()
   rc = lib.xla_amd_qmm_quantize_per_token(None, None, None, None, 1, 1, 0, 0, 0, None)

@@ -17,7 +17,7 @@ OVERFLOW_SATURATE, OVERFLOW_WRAP = 0, 1
 W_NK, W_SCN = 0, 1
 QDT_I8, QDT_U8, QDT_I16, QDT_I32 = 0, 1, 2, 3
 KERNEL_GENERIC, KERNEL_SKINNY_MFMA, KERNEL_W8A8_MFMA, KERNEL_W8A8_GENERIC, KERNEL_WEIGHT_ONLY_GEMM = 0, 1, 2, 3, 4
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 
@@ -29,7 +29,8 @@ SIGNATURES = {
     "xla_amd_qmm_last_error": (ctypes.c_char_p, []),
     "xla_amd_qmm_packed_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_int]),
     "xla_amd_qmm_pack_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
-    "xla_amd_qmm_tiled_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_int]),
+    "xla_amd_qmm_tile_group": (_c_int, [_c_i64, _c_i64, _c_i64, _c_int]),
+    "xla_amd_qmm_tiled_bytes": (ctypes.c_size_t, [_c_i64, _c_i64, _c_i64, _c_int]),
     "xla_amd_qmm_tile_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
     "xla_amd_qmm_untile_weight": (_c_int, [_c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_vp]),
     "xla_amd_qmm_weight_only_skinny": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),

@@ -45,6 +45,7 @@ SOURCES = [
 TIMELINE_LIB_PATH = os.path.join(PKG_DIR, "libxla_amd_qmm_timeline.so")
 TIMELINE_UNIT = ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=1", "-DQMM_SKINNY_TIMELINE"], "qmm_skinny_bf16_timeline.o")
 TIMELINE_REPLACES = "qmm_skinny_bf16.o"
+DIAG_UNIT = ("qmm_diag.hip", [], "qmm_diag.o")  # diagnostic kernels: the diagnostic library only
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -111,13 +112,14 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     return obj, kernels
 
   with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-    results = list(ex.map(compile_one, SOURCES + [TIMELINE_UNIT]))
+    results = list(ex.map(compile_one, SOURCES + [TIMELINE_UNIT, DIAG_UNIT]))
+  diag_obj, diag_kernels = results.pop()
   timeline_obj, timeline_kernels = results.pop()
   objs = [r[0] for r in results]
   kernels = [k for r in results for k in r[1]]
   with open(RESOURCES_PATH, "w") as f:
     json.dump(kernels, f, indent=1)
-  spilling = [k for k in kernels + timeline_kernels if k.get("scratch_bytes_per_lane", 0) > 0]
+  spilling = [k for k in kernels + timeline_kernels + diag_kernels if k.get("scratch_bytes_per_lane", 0) > 0]
   if spilling:
     raise RuntimeError("kernels with a scratch frame (register spills):\n" +
                        "\n".join("  %s: %s (%d bytes per lane, %d VGPRs)" % (k["unit"], k["kernel"], k["scratch_bytes_per_lane"],
@@ -127,7 +129,7 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
   os.replace(tmp, LIB_PATH)
   tmp = TIMELINE_LIB_PATH + ".tmp"
   _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] +
-       [timeline_obj if os.path.basename(o) == TIMELINE_REPLACES else o for o in objs])
+       [timeline_obj if os.path.basename(o) == TIMELINE_REPLACES else o for o in objs] + [diag_obj])
   os.replace(tmp, TIMELINE_LIB_PATH)
   return LIB_PATH
 

@@ -42,9 +42,41 @@ extern "C" size_t xla_amd_qmm_packed_bytes(int64_t N, int64_t K, int bits) {
   return 0;
 }
 
-extern "C" size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int bits) {
+// Channels per group of the tiled copy.  A wave of the streaming kernel owns one group over all of K
+// (or, with KW waves splitting K, a KW-th of it), and a launch should fill the chip's 256 compute units
+// x 4 waves in whole rounds: 14336 channels in groups of 16 are 896 waves = 224 workgroups, 32 compute
+// units idle for the whole launch; in groups of 14 they are 1024 waves on all 256.  So per-channel int8
+// weights are tiled in groups of 16, 14, 12 or 10 channels, whichever fills the last round best (the
+// wider group unless a narrower one gains 4 % or more); blockwise and int4 weights keep 16.
+extern "C" int xla_amd_qmm_tile_group(int64_t N, int64_t K, int64_t C, int bits) {
+  if (N <= 0 || K <= 0) return 0;
+  if (C <= 0) C = K;
+  if (bits != 8 || C != K || N < 4096) return 16;
+  auto fill = [&](int64_t g) -> double {
+    const int64_t groups = (N + g - 1) / g;
+    const double used = (double)N / (double)(groups * g);  // channels past N in the last group
+    int64_t kw = 1;
+    if (groups * 2 <= 1024) kw = 2;
+    if (groups * 4 <= 1024) kw = 4;
+    const int64_t waves = groups * kw;
+    if (waves <= 1024) return used * (double)waves / 1024.0;
+    // more than one round of four-wave workgroups: eight computing waves per workgroup, 2048 per round
+    const int64_t rounds = (groups + 2047) / 2048;
+    return used * (double)groups / (double)(rounds * 2048);
+  };
+  int best = 16;
+  double best_fill = fill(16);
+  for (int g : {14, 12, 10}) {
+    const double f = fill(g);
+    if (f >= best_fill + 0.04) { best = g; best_fill = f; }
+  }
+  return best;
+}
+
+extern "C" size_t xla_amd_qmm_tiled_bytes(int64_t N, int64_t K, int64_t C, int bits) {
   if (N <= 0 || K <= 0 || K % 128 != 0 || (bits != 4 && bits != 8)) return 0;
-  const size_t rows = (size_t)((N + 15) / 16) * 16;
+  const int64_t g = xla_amd_qmm_tile_group(N, K, C, bits);
+  const size_t rows = (size_t)((N + g - 1) / g) * (size_t)g;
   return bits == 8 ? rows * (size_t)K : rows * (size_t)K / 2;
 }
 
@@ -68,10 +100,11 @@ int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int64_t C, int bits, in
   // (measured with cold weights at M = 32: 4096 x 14336 25.5 -> 17.8 us; with fewer than 8 rows the second kernel
   // costs more than the copies saved, and so it does with K = 4096 unless the output is narrow and x two tiles
   // high: 1024 x 4096 at M = 32 8.6 -> 7.5 us, 2048 x 4096 8.8 -> 8.4, but 4096 x 4096 9.4 -> 9.9)
-  const int64_t cols = (N + 63) / 64;
+  const int64_t g_ch = xla_amd_qmm_tile_group(N, K, C, bits);
+  const int64_t cols = ((N + g_ch - 1) / g_ch + 3) / 4;  // workgroups of four channel groups
   if (M < 8 || K < 4096) return 1;
   if (K < 8192 && !(M > 16 && cols <= 16)) return 1;
-  if (cols >= 128) return 1;  // enough workgroups of 64 channels already
+  if (cols >= 128) return 1;  // enough workgroups of four channel groups already
   const int64_t steps = K / ks;
   int64_t slices = 256 / cols;
   if (slices > steps / 2) slices = steps / 2;  // at least two steps per slice

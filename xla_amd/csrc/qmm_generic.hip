@@ -154,20 +154,30 @@ qmm_pack_kernel(const int8_t* __restrict__ w, uint32_t* __restrict__ packed, int
 }
 
 // Tiled copy for the streaming kernel: one thread writes the 16 bytes that one
-// lane of one 1 KB load will receive.
-__global__ void __launch_bounds__(256)
-qmm_tile_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ tiled, int64_t N, int64_t K,
-                int src_layout, int bits, int64_t total) {
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= total) return;
-  const int chunks = bits == 8 ? 128 : 64;  // 16-byte chunks per block
+// lane of one load will receive.  G channels per group (16, or fewer for some
+// per-channel int8 weights): a block holds, for each half h and quarter q of its
+// 128 columns, G rows of 16 bytes.
+struct TileIndex {
+  int64_t n, k0;
+};
+__device__ __forceinline__ TileIndex qmm_tile_index(int64_t idx, int64_t K, int bits, int G) {
+  const int halves = bits == 8 ? 2 : 1;
+  const int chunks = halves * 4 * G;  // 16-byte chunks per block
   const int c = (int)(idx % chunks);
   const int64_t blk = idx / chunks;
   const int64_t n_blk = K / 128;
-  const int64_t t = blk % n_blk, g = blk / n_blk;
-  const int l = c & 63, h = c >> 6;
-  const int64_t n = 16 * g + (l & 15);
-  const int64_t k0 = 128 * t + 32 * (l >> 4) + 16 * h;
+  const int64_t t = blk % n_blk, p = blk / n_blk;
+  const int h = c / (4 * G), q = (c % (4 * G)) / G, r = c % G;
+  return TileIndex{(int64_t)G * p + r, 128 * t + 32 * q + 16 * h};
+}
+
+__global__ void __launch_bounds__(256)
+qmm_tile_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ tiled, int64_t N, int64_t K,
+                int src_layout, int bits, int G, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const TileIndex ti = qmm_tile_index(idx, K, bits, G);
+  const int64_t n = ti.n, k0 = ti.k0;
   auto at = [&](int64_t k) -> int { return src_layout == XLA_AMD_W_NK ? w[n * K + k] : w[k * N + n]; };
   i32x4 v = {0, 0, 0, 0};
   if (n < N) {
@@ -189,6 +199,11 @@ qmm_tile_kernel(const int8_t* __restrict__ w, i32x4* __restrict__ tiled, int64_t
   tiled[idx] = v;
 }
 
+// 16-byte chunks of the tiled copy (one thread each)
+static int64_t qmm_tile_chunks(int64_t N, int64_t K, int bits, int G) {
+  return ((N + G - 1) / G) * (K / 128) * (bits == 8 ? 8 : 4) * G;
+}
+
 extern "C" int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, int64_t C, int64_t N,
                                        int src_layout, int bits, void* stream) {
   if (!w || !tiled) return qmm_fail(XLA_AMD_QMM_EINVAL, "tile_weight: null pointer");
@@ -198,11 +213,12 @@ extern "C" int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, 
     return qmm_fail(XLA_AMD_QMM_EINVAL, "tile_weight: bad layout %d", src_layout);
   const int64_t K = S * C;
   if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "tile_weight: K=%lld not a multiple of 128", (long long)K);
-  const int64_t total = ((N + 15) / 16) * (K / 128) * (bits == 8 ? 128 : 64);
+  const int G = xla_amd_qmm_tile_group(N, K, S == 1 ? K : C, bits);
+  const int64_t total = qmm_tile_chunks(N, K, bits, G);
   const int64_t blocks = (total + 255) / 256;
   if (blocks > 0x7fffffffLL) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "tile_weight: weight too large");
   hipLaunchKernelGGL(qmm_tile_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, w,
-                     (i32x4*)tiled, N, K, src_layout, bits, total);
+                     (i32x4*)tiled, N, K, src_layout, bits, G, total);
   return QMM_CHECK_LAUNCH("tile_weight launch");
 }
 
@@ -210,18 +226,12 @@ extern "C" int xla_amd_qmm_tile_weight(const int8_t* w, void* tiled, int64_t S, 
 // the 16 (bits 8) or 32 (bits 4) weights they hold back into the operator's layout.
 __global__ void __launch_bounds__(256)
 qmm_untile_kernel(const i32x4* __restrict__ tiled, int8_t* __restrict__ w, int64_t N, int64_t K,
-                  int dst_layout, int bits, int64_t total) {
+                  int dst_layout, int bits, int G, int64_t total) {
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
-  const int chunks = bits == 8 ? 128 : 64;
-  const int c = (int)(idx % chunks);
-  const int64_t blk = idx / chunks;
-  const int64_t n_blk = K / 128;
-  const int64_t t = blk % n_blk, g = blk / n_blk;
-  const int l = c & 63, h = c >> 6;
-  const int64_t n = 16 * g + (l & 15);
+  const TileIndex ti = qmm_tile_index(idx, K, bits, G);
+  const int64_t n = ti.n, k0 = ti.k0;
   if (n >= N) return;
-  const int64_t k0 = 128 * t + 32 * (l >> 4) + 16 * h;
   const i32x4 v = tiled[idx];
   auto put = [&](int64_t k, int val) {
     if (dst_layout == XLA_AMD_W_NK) w[n * K + k] = (int8_t)val;
@@ -246,11 +256,12 @@ extern "C" int xla_amd_qmm_untile_weight(const void* tiled, int8_t* w, int64_t S
     return qmm_fail(XLA_AMD_QMM_EINVAL, "untile_weight: bad layout %d", dst_layout);
   const int64_t K = S * C;
   if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "untile_weight: K=%lld not a multiple of 128", (long long)K);
-  const int64_t total = ((N + 15) / 16) * (K / 128) * (bits == 8 ? 128 : 64);
+  const int G = xla_amd_qmm_tile_group(N, K, S == 1 ? K : C, bits);
+  const int64_t total = qmm_tile_chunks(N, K, bits, G);
   const int64_t blocks = (total + 255) / 256;
   if (blocks > 0x7fffffffLL) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "untile_weight: weight too large");
   hipLaunchKernelGGL(qmm_untile_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const i32x4*)tiled, w, N, K, dst_layout, bits, total);
+                     (const i32x4*)tiled, w, N, K, dst_layout, bits, G, total);
   return QMM_CHECK_LAUNCH("untile_weight launch");
 }
 

@@ -11,6 +11,7 @@ struct SkinnyArgs {
   const void* zp;
   void* out;
   int M, N, K, C;  // M = rows of this pass (<= 16*MT)
+  int G;           // channels per group of the tiled weight (xla_amd_qmm_tile_group)
   int scale_dt, zp_dt, out_dt;
   int dot_dt;    // dtype the dot product is rounded to before it is scaled (per-channel only)
   int store_dt;  // dtype of the stored tensor (out_dt, or a final cast of it)

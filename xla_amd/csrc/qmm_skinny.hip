@@ -182,7 +182,16 @@ qmm_skinny_kernel(SkinnyArgs a) {
   const int k_begin = (int)blockIdx.y * a.k_per_slice;
   const int K = min(a.k_per_slice, ldk - k_begin);
   const int N = a.N, M = a.M, C = a.C == a.K ? K : a.C;  // per-channel: the slice is the one block
-  const int n_wave = blockIdx.x * (16 * RW) + 16 * rw;  // first channel of this wave
+  // This wave's channels: group grp_u of G channels (G = 16, or the narrower group of some per-channel int8
+  // weights, see xla_amd_qmm_tile_group), ch_lo .. ch_hi - 1.  MFMA row 0 is channel n_wave, the four-aligned
+  // channel at or below ch_lo, so that a lane's four results stay four-aligned for its stores; the rows below
+  // ch_lo (two at most) and from ch_hi on are fed some other row's weights and their results are dropped.
+  constexpr bool kGrouped = RED == kRedRaw && BITS == 8;
+  const int G = kGrouped ? a.G : 16;
+  const int grp_u = blockIdx.x * RW + rw;
+  const int ch_lo = grp_u * G, ch_hi = min(ch_lo + G, N);
+  const int n_wave = ch_lo & ~3;
+  const int row_off = ch_lo - n_wave;
   const int x_dt = XT;
   const int scale_dt = UNI ? XT : a.scale_dt, zp_dt = UNI ? XT : a.zp_dt, out_dt = UNI ? XT : a.out_dt;
   const int dot_dt = UNI ? XT : a.dot_dt, store_dt = UNI ? XT : a.store_dt;
@@ -194,9 +203,12 @@ qmm_skinny_kernel(SkinnyArgs a) {
   // along K, so a wave streams one contiguous region.  Lane l of a 1 KB load
   // takes bytes [16 l, 16 l + 16): its own operand fragment.
   const int n_blk = K / 128;                                    // blocks of this slice per channel group
-  const int groups = (N + 15) / 16;
-  const int my_group = min((int)blockIdx.x * RW + rw, groups - 1);  // tail groups re-read the last one
-  const uint8_t* const w_base = a.w + ((size_t)my_group * (ldk / 128) + k_begin / 128) * BLK + lane * 16;
+  const int groups = (N + G - 1) / G;
+  const int my_group = min(grp_u, groups - 1);  // tail groups re-read the last one
+  const int blk_bytes = kGrouped ? G * 128 : BLK;                // bytes of one (G channels x 128 columns) weight block
+  const int half_bytes = G * 64;                                 // (bits 8) second half of a block: columns 16 .. 31 of every quarter
+  const int srow = min(max(r - row_off, 0), G - 1);              // row of the block that this lane's MFMA row reads
+  const uint8_t* const w_base = a.w + ((size_t)my_group * (ldk / 128) + k_begin / 128) * blk_bytes + (g * G + srow) * 16;
   const char* const x_base = (const char*)a.x + (size_t)k_begin * XB;
   // x: copied global -> LDS without passing registers (global_load_lds_dwordx4:
   // lane l of an instruction lands at base + 16 l), 1 KB of one row per
@@ -218,10 +230,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
   auto load_sub = [&](auto pc, int s, auto tc) __attribute__((always_inline)) {
     constexpr int p = pc, t = tc;
     const int blk = min((s * KW + kw) * SUB + t, n_blk - 1);
-    const uint8_t* const wp = w_base + (size_t)blk * BLK;
+    const uint8_t* const wp = w_base + (size_t)blk * blk_bytes;
     qmm_static_for<kLoadsPerSub>([&](auto hc) {
       constexpr int h = hc;
-      wreg[p][kLoadsPerSub * t + h] = __builtin_nontemporal_load((const i32x4*)(wp + h * 1024));
+      wreg[p][kLoadsPerSub * t + h] = __builtin_nontemporal_load((const i32x4*)(wp + h * half_bytes));
     });
   };
   auto load_regs = [&](auto pc, int s) __attribute__((always_inline)) {
@@ -680,14 +692,14 @@ qmm_skinny_kernel(SkinnyArgs a) {
         constexpr int mt = mc;
         const int m = 16 * mt + r;
         const int n = n_wave + 4 * g;
-        if (m < M && n < N) {
+        if (m < M && n + 3 >= ch_lo && n < ch_hi) {
           float* p = a.part + ((size_t)slice * M + m) * N + n;
           // (the slice's dot product: with int4 weights the affine map is undone with the slice's own row sum)
           const float xsv = NEEDXS ? xs[mt][0] : 0.f;
           const f32x4 t = {true_dot(acc[mt][0] + accb[mt][0], xsv), true_dot(acc[mt][1] + accb[mt][1], xsv),
                            true_dot(acc[mt][2] + accb[mt][2], xsv), true_dot(acc[mt][3] + accb[mt][3], xsv)};
-          if ((N & 3) == 0) *(f32x4*)p = t;
-          else for (int v = 0; v < 4; ++v) if (n + v < N) p[v] = t[v];
+          if ((N & 3) == 0 && n >= ch_lo && n + 3 < ch_hi) *(f32x4*)p = t;
+          else for (int v = 0; v < 4; ++v) if (n + v >= ch_lo && n + v < ch_hi) p[v] = t[v];
           if constexpr (NEEDXS) {
             if (n_wave == 0 && g == 0) a.part_xs[(size_t)slice * M + m] = xs[mt][0];
           }
@@ -704,7 +716,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
     constexpr int mt = mc;
     const int m = 16 * mt + r;
     const int n = n_wave + 4 * g;
-    if (m < M && n < N) {
+    if (m < M && n + 3 >= ch_lo && n < ch_hi) {
       constexpr float kBlockFactor = (RED != kRedRaw && BITS == 4 && kMfma) ? 16.0f : 1.0f;  // see block_epilogue
       if constexpr (RED != kRedRaw) {
         if (a.slices > 1) {
@@ -728,7 +740,7 @@ qmm_skinny_kernel(SkinnyArgs a) {
       // (a store dtype narrower than out_dt is the caller's final cast: one more rounding, done by the conversion)
       const int st = store_dt;
       const size_t idx = (size_t)m * N + n;
-      if ((N & 3) == 0) {  // 4 consecutive channels: one aligned 8- or 16-byte store
+      if ((N & 3) == 0 && n >= ch_lo && n + 3 < ch_hi) {  // 4 consecutive channels of this wave: one aligned 8- or 16-byte store
         if (st == XLA_AMD_DT_F32) {
           *(f32x4*)((float*)a.out + idx) = f32x4{o0, o1, o2, o3};
         } else {
@@ -740,10 +752,10 @@ qmm_skinny_kernel(SkinnyArgs a) {
           *(i32x2*)((uint16_t*)a.out + idx) = i32x2{(int)(h0 | (h1 << 16)), (int)(h2 | (h3 << 16))};
         }
       } else {
-        qmm_store(a.out, idx, o0, st);
-        if (n + 1 < N) qmm_store(a.out, idx + 1, o1, st);
-        if (n + 2 < N) qmm_store(a.out, idx + 2, o2, st);
-        if (n + 3 < N) qmm_store(a.out, idx + 3, o3, st);
+        if (n >= ch_lo) qmm_store(a.out, idx, o0, st);
+        if (n + 1 >= ch_lo && n + 1 < ch_hi) qmm_store(a.out, idx + 1, o1, st);
+        if (n + 2 >= ch_lo && n + 2 < ch_hi) qmm_store(a.out, idx + 2, o2, st);
+        if (n + 3 < ch_hi) qmm_store(a.out, idx + 3, o3, st);
       }
     }
   });
@@ -767,7 +779,9 @@ int launch_kernel(const SkinnyArgs& a, hipStream_t stream) {
 #endif
     const int rc = qmm_set_max_lds((const void*)kern, kMaxLds, lds_set, "weight_only_skinny hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
-    const unsigned blocks = (unsigned)((a.N + 16 * Cfg::RW - 1) / (16 * Cfg::RW));
+    const int g_ch = (RED == kRedRaw && BITS == 8) ? a.G : 16;
+    const int groups = (a.N + g_ch - 1) / g_ch;
+    const unsigned blocks = (unsigned)((groups + Cfg::RW - 1) / Cfg::RW);
     const int steps = (a.k_per_slice + Cfg::KS - 1) / Cfg::KS;
     constexpr int kScl = skinny_scale_bytes<Cfg, XT, MT, RED, KW>();
     int lds = Cfg::lds_bytes(steps, kSlots) + kScl;
@@ -814,7 +828,9 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
   const bool perch = a.C == a.K;
   const bool can_split = perch || (KS % a.C == 0);
   const int steps = (a.k_per_slice + KS - 1) / KS;  // of one workgroup
-  auto workgroups = [&](int kw_) { return ((int64_t)a.N + 64 / kw_ - 1) / (64 / kw_) * a.slices; };  // K slices multiply them too
+  const int g_ch = (perch && BITS == 8) ? a.G : 16;                    // channels per group of the tiled weight
+  const int64_t groups = ((int64_t)a.N + g_ch - 1) / g_ch;
+  auto workgroups = [&](int kw_) { return (groups + 4 / kw_ - 1) / (4 / kw_) * a.slices; };  // K slices multiply them too
   int kw = 1;
   if (can_split) {
     if (workgroups(2) <= kComputeUnits && steps >= 2 && SkinnyCfg<XT, BITS, MT, 2>::kFits) kw = 2;
@@ -923,6 +939,7 @@ extern "C" int xla_amd_qmm_weight_only_skinny(const void* x, const void* w_tiled
     a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.out_dt = out_dt;
     a.dot_dt = dot_dt; a.store_dt = store_dt;
     a.k_per_slice = (int)K; a.slices = 1; a.part = nullptr; a.part_xs = nullptr; a.part_z = nullptr;
+    a.G = xla_amd_qmm_tile_group(N, K, C, bits);
     int rc;
     if (x_dt == XLA_AMD_DT_BF16) rc = qmm_skinny_launch_bf16(a, bits, zp != nullptr, (hipStream_t)stream);
     else if (x_dt == XLA_AMD_DT_F16) rc = qmm_skinny_launch_f16(a, bits, zp != nullptr, (hipStream_t)stream);

@@ -50,6 +50,7 @@ struct WoGemmArgs {
   float* part;         // [split][M][N] partial dot products (split > 1)
   float* part_xs;      // [split][M] partial row sums of x (split > 1, zero point)
   int M, N, K;
+  int G;               // channels per group of the tiled weight (xla_amd_qmm_tile_group)
   int k_per_split;     // columns per K slice (a multiple of 128)
   int split;
   int scale_dt, zp_dt, dot_dt, out_dt, store_dt;
@@ -137,6 +138,33 @@ __device__ __forceinline__ void wo_store4(void* out, int m, int n, int N, const 
   }
 }
 
+// Stores the first cnt (1 .. 4) of four consecutive channels of row m starting at channel n, n even: in
+// pairs where the row length allows it (channel groups narrower than 16 start on even, not on
+// four-aligned channels, and their last lane holds two channels).
+__device__ __forceinline__ void wo_store_some(void* out, int m, int n, int N, int cnt, const float o[4], int store_dt) {
+  const size_t idx = (size_t)m * N + n;
+  if ((N & 1) == 0) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      if (cnt >= 2 * h + 2) {
+        if (store_dt == XLA_AMD_DT_F32) {
+          typedef float f32x2_t __attribute__((ext_vector_type(2)));
+          *(f32x2_t*)((float*)out + idx + 2 * h) = f32x2_t{o[2 * h], o[2 * h + 1]};
+        } else {
+          *(uint32_t*)((uint16_t*)out + idx + 2 * h) = store_dt == XLA_AMD_DT_BF16 ? qmm_f32x2_to_bf16x2(o[2 * h], o[2 * h + 1])
+                                                                                  : qmm_f32x2_to_f16x2(o[2 * h], o[2 * h + 1]);
+        }
+      } else if (cnt == 2 * h + 1) {
+        qmm_store(out, idx + 2 * h, o[2 * h], store_dt);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (v < cnt) qmm_store(out, idx + v, o[v], store_dt);
+  }
+}
+
 // The same epilogue and store when every dtype is bf16 and there is no zero point: two
 // values per conversion, and the rounded product is already the stored bit pattern.
 __device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, int N, const uint32_t sraw[4], f32x4 dot) {
@@ -152,7 +180,7 @@ __device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, in
 
 // One unit of work: a tile of rows x channels over one K slice.
 struct WoItem {
-  int m0, n0, ks, k_begin, steps, n_chunks, rows;
+  int m0, g0, ks, k_begin, steps, n_chunks, rows;  // g0: first channel group of the column tile
 };
 
 // The kernel is persistent: workgroup b takes the work items b, b + gridDim.x, ... one after the
@@ -164,15 +192,16 @@ __global__ void __launch_bounds__((kComputeWaves + kCopyWaves) * 64)
 qmm_wo_gemm_kernel(WoGemmArgs a) {
   using Cfg = WoCfg<MT, NG>;
   constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE, CS = Cfg::CS;
-  constexpr int BN = 64 * NG;  // channels per workgroup: NG groups of 16 per computing wave
+  constexpr int GPT = 4 * NG;  // channel groups per workgroup: NG per computing wave (groups of a.G channels, 16 or fewer)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
-  const int M = a.M, N = a.N, K = a.K;
-  const int tiles_n = (N + BN - 1) / BN;
+  const int M = a.M, N = a.N, K = a.K, G = a.G;
+  const int groups = (N + G - 1) / G;
+  const int tiles_n = (groups + GPT - 1) / GPT;
   const int tiles = tiles_n * ((M + BM - 1) / BM);
   const int n_items = tiles * a.split;
   // item -> (K slice, row tile, column tile), column tiles fastest: workgroups that run together share x rows
@@ -181,7 +210,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     const int tile = it % tiles;
     w.ks = it / tiles;
     w.m0 = (tile / tiles_n) * BM;
-    w.n0 = (tile % tiles_n) * BN;
+    w.g0 = (tile % tiles_n) * GPT;
     w.k_begin = w.ks * a.k_per_split;
     w.steps = (min(K, w.k_begin + a.k_per_split) - w.k_begin) / 128;  // >= 1
     w.n_chunks = (w.steps + CS - 1) / CS;
@@ -229,24 +258,27 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   }
 
   // ---- computing waves ----
-  // wave w owns the channel groups (n0/16 + w*NG) .. + NG-1 of the item's column tile
+  // wave w owns the channel groups g0 + w*NG .. + NG-1 of the item's column tile.  Group p holds the
+  // channels G p .. G p + G - 1 in MFMA rows 0 .. G - 1; the rows from G on (groups narrower than 16) read
+  // the group's last row again and their results are dropped.
   const int n_blk = K / 128;  // blocks per channel group in the tiled weight
-  const int groups = (N + 15) / 16;
+  const int blk_bytes = G * 128, half_bytes = G * 64;
   constexpr int P = Cfg::P;
   const uint8_t* wp[NG];
   i32x4 wreg[P][NG][2];  // ring slot s % P holds the block of step s
   auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      const int grp = min(w.n0 / 16 + wave * NG + gi, groups - 1);  // groups past N re-read the last one
-      wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * 2048 + lane * 16;
+      const int grp_u = w.g0 + wave * NG + gi;
+      const int grp = min(grp_u, groups - 1);  // groups past N re-read the last one
+      wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * blk_bytes + (g * G + min(r, G - 1)) * 16;
     });
   };
   auto load_half = [&](int blk, auto slotc, auto hc) __attribute__((always_inline)) {
     constexpr int slot = slotc, h = hc;
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      wreg[slot][gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * 2048 + h * 1024));
+      wreg[slot][gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * blk_bytes + h * half_bytes));
     });
   };
   // the first P blocks of an item (a block past the end of a short item is the last one again: never used)
@@ -346,7 +378,14 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     }
 
     // ---- results: four consecutive channels of one row per lane ----
-    const int m0 = done.m0, n0 = done.n0;
+    const int m0 = done.m0;
+    // channels of this lane for group gi of its wave: n .. n + cnt - 1 (cnt <= 4; computed where they are
+    // used: the 128 x 256 tile has no register to keep them in)
+    const int g_first = done.g0 + wave * NG;
+    auto chan = [&](int gi, int& n, int& cnt) __attribute__((always_inline)) {
+      n = (g_first + gi) * G + 4 * g;
+      cnt = min(min(G - 4 * g, N - n), 4);
+    };
     if (a.split == 1) {
       const WoDts<XT, UNI> dts(a);
       // scales (and zero points) of this lane's channels first, all at once: loads inside the
@@ -354,7 +393,9 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       uint32_t sraw[NG][4], zraw[NG][4];
       qmm_static_for<NG>([&](auto gc) {
         constexpr int gi = gc;
-        const int n = min(n0 + (wave * NG + gi) * 16 + 4 * g, N - 1);
+        int n, cnt;
+        chan(gi, n, cnt);
+        n = min(n, N - 1);
         wo_load4_raw(a.scale, n, N, dts.scale_dt, sraw[gi]);
         if constexpr (HASZP) wo_load4_raw(a.zp, n, N, dts.zp_dt, zraw[gi]);
       });
@@ -366,14 +407,21 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
           const int m = m0 + 16 * mt + r;
           qmm_static_for<NG>([&](auto gc) {
             constexpr int gi = gc;
-            const int n = n0 + (wave * NG + gi) * 16 + 4 * g;
-            if (m < M && n < N) {
-              if constexpr (kVec && UNI && !HASZP && XT == XLA_AMD_DT_BF16) {
-                wo_finish_store_bf16(a.out, m, n, N, sraw[gi], acc[gi][mt]);
+            int n, cnt;
+            chan(gi, n, cnt);
+            if (m < M && cnt > 0) {
+              if (kVec && cnt == 4 && (n & 3) == 0) {  // four channels, four-aligned: one store
+                if constexpr (kVec && UNI && !HASZP && XT == XLA_AMD_DT_BF16) {
+                  wo_finish_store_bf16(a.out, m, n, N, sraw[gi], acc[gi][mt]);
+                } else {
+                  float o[4];
+                  wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, XT, o);
+                  wo_store4<kVec>(a.out, m, n, N, o, dts.store_dt);
+                }
               } else {
                 float o[4];
                 wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, XT, o);
-                wo_store4<kVec>(a.out, m, n, N, o, dts.store_dt);
+                wo_store_some(a.out, m, n, N, cnt, o, dts.store_dt);
               }
             }
           });
@@ -385,20 +433,21 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       const bool vec = (N & 3) == 0;
       qmm_static_for<NG>([&](auto gc) {
         constexpr int gi = gc;
-        const int n = n0 + (wave * NG + gi) * 16 + 4 * g;
+        int n, cnt;
+        chan(gi, n, cnt);
         qmm_static_for<MT>([&](auto mc) {
           constexpr int mt = mc;
           const int m = m0 + 16 * mt + r;
-          if (m < M && n < N) {
+          if (m < M && cnt > 0) {
             float* p = a.part + ((size_t)done.ks * M + m) * N + n;
-            if (vec) *(f32x4*)p = acc[gi][mt];
-            else for (int v = 0; v < 4; ++v) if (n + v < N) p[v] = acc[gi][mt][v];
+            if (vec && cnt == 4 && (n & 3) == 0) *(f32x4*)p = acc[gi][mt];
+            else for (int v = 0; v < 4; ++v) if (v < cnt) p[v] = acc[gi][mt][v];
           }
         });
       });
       if constexpr (HASZP) {
         // partial row sums of x: once per row tile and K slice (the first column tile's first wave, channel lanes 0..15)
-        if (n0 == 0 && wave == 0 && g == 0) {
+        if (done.g0 == 0 && wave == 0 && g == 0) {
           qmm_static_for<MT>([&](auto mc) {
             constexpr int mt = mc;
             const int m = m0 + 16 * mt + r;
@@ -427,7 +476,8 @@ int cu_count() {
 template <int XT, int MT, int NG>
 int launch(const WoGemmArgs& a, hipStream_t stream) {
   using Cfg = WoCfg<MT, NG>;
-  const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * ((a.N + 64 * NG - 1) / (64 * NG)) * a.split;
+  const int64_t groups = ((int64_t)a.N + a.G - 1) / a.G;
+  const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * ((groups + 4 * NG - 1) / (4 * NG)) * a.split;
   const int steps = a.k_per_split / 128;
   // one workgroup per compute unit (its LDS and registers leave room for no second one); each walks its share of the items
   const int cus = cu_count();
@@ -559,9 +609,11 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
   p.mt = M <= 64 ? 4 : 8;
   const int64_t bm = 16 * p.mt;
   const int64_t tiles_m = (M + bm - 1) / bm;
+  const int64_t g_ch = xla_amd_qmm_tile_group(N, K, K, 8);
+  const int64_t groups = (N + g_ch - 1) / g_ch;  // a column tile is 4 * ng channel groups
   p.ng = 4;
-  if ((tiles_m * ((N + 255) / 256) < 192 && N > 128) || (has_zp && p.mt == 8)) p.ng = 2;
-  const int64_t tiles = tiles_m * ((N + 64 * p.ng - 1) / (64 * p.ng));
+  if ((tiles_m * ((groups + 15) / 16) < 192 && N > 128) || (has_zp && p.mt == 8)) p.ng = 2;
+  const int64_t tiles = tiles_m * ((groups + 4 * p.ng - 1) / (4 * p.ng));
   int64_t split = 1;
   if (tiles < 192) split = (256 + tiles - 1) / tiles;
   const int64_t blocks = K / 128;
@@ -634,6 +686,7 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
       SkinnyArgs k;
       k.x = x; k.w = (const uint8_t*)w_tiled; k.scale = scale; k.zp = zp; k.out = out;
       k.M = (int)M; k.N = (int)N; k.K = (int)K; k.C = (int)C;
+      k.G = xla_amd_qmm_tile_group(N, K, C, bits);
       k.scale_dt = scale_dt; k.zp_dt = zp ? zp_dt : x_dt; k.out_dt = out_dt; k.dot_dt = dot_dt; k.store_dt = store_dt;
       k.k_per_slice = per; k.slices = slices;
       k.part = (float*)workspace;
@@ -653,7 +706,7 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
       WoGemmArgs f;
       f.x = x; f.w = (const uint8_t*)w_tiled; f.scale = scale; f.zp = zp; f.out = out;
       f.part = k.part; f.part_xs = k.part_xs;
-      f.M = (int)M; f.N = (int)N; f.K = (int)K; f.k_per_split = per; f.split = slices;
+      f.M = (int)M; f.N = (int)N; f.K = (int)K; f.G = k.G; f.k_per_split = per; f.split = slices;
       f.scale_dt = scale_dt; f.zp_dt = zp ? zp_dt : x_dt; f.dot_dt = dot_dt; f.out_dt = out_dt; f.store_dt = store_dt;
       const int64_t threads = M * ((N + 3) / 4);
       hipLaunchKernelGGL(qmm_wo_gemm_finish_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
@@ -685,6 +738,7 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
   a.x = x; a.w = (const uint8_t*)w_tiled; a.scale = scale; a.zp = zp; a.out = out;
   a.part = nullptr; a.part_xs = nullptr;
   a.M = (int)M; a.N = (int)N; a.K = (int)K;
+  a.G = xla_amd_qmm_tile_group(N, K, K, 8);
   a.k_per_split = p.k_per_split; a.split = p.split;
   a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.dot_dt = dot_dt; a.out_dt = out_dt; a.store_dt = store_dt;
   if (p.split > 1) {

@@ -143,9 +143,10 @@ def _relayout(w: torch.Tensor, bits: int, layout: int, kind: str) -> torch.Tenso
     s, c, n = w.shape
     k = s * c
   lib = _lib.load()
-  size_fn, copy_fn = ((lib.xla_amd_qmm_tiled_bytes, lib.xla_amd_qmm_tile_weight) if kind == "tiled" else
-                      (lib.xla_amd_qmm_packed_bytes, lib.xla_amd_qmm_pack_weight))
-  nbytes = size_fn(n, k, bits)
+  if kind == "tiled":
+    copy_fn, nbytes = lib.xla_amd_qmm_tile_weight, lib.xla_amd_qmm_tiled_bytes(n, k, c, bits)
+  else:
+    copy_fn, nbytes = lib.xla_amd_qmm_pack_weight, lib.xla_amd_qmm_packed_bytes(n, k, bits)
   if nbytes == 0:
     raise RuntimeError(f"xla_amd: cannot re-lay out weight of shape {tuple(w.shape)} to {bits} bits ({kind})")
   out = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
@@ -165,7 +166,7 @@ def _packed_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
 
 
 def _tiled_weight(w: torch.Tensor, bits: int, layout: int) -> torch.Tensor:
-  """Tiled copy of w for the streaming kernel (blocks of 16 channels x 128 columns in MFMA operand order).
+  """Tiled copy of w for the streaming kernel (blocks of a channel group x 128 columns in MFMA operand order).
 
   The copy is made once per weight tensor and reused while the tensor is alive
   and unmodified (same object, same storage pointer, same version counter); it
@@ -474,7 +475,7 @@ def weight_only_tiled_rocm(x, w_tiled, scaler, zero_point, out_features, block_s
   k = x.shape[-1]
   c = k if block_size == -1 else block_size
   bits = 4 if int4_weight else 8
-  need = _lib.load().xla_amd_qmm_tiled_bytes(out_features, k, bits)
+  need = _lib.load().xla_amd_qmm_tiled_bytes(out_features, k, c, bits)
   assert need > 0 and w_tiled.numel() * w_tiled.element_size() == need, (
       f"tiled weight of {w_tiled.numel() * w_tiled.element_size()} bytes does not belong to a "
       f"[{out_features}, {k}] weight of {bits} bits")
