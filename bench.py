@@ -35,7 +35,19 @@ BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA (2.5 PFLOP/s)
 PREWARM_MS = 50.0  # untimed graph replays before each timed region (sustained clocks)
 
 N_OUT, K_IN = 14336, 4096
-TRAFFIC_BYTES_PER_LAUNCH = 60.4e6  # decode GEMV M=16, see profiles/skinny_gemv_cfg2_m16_hbm_traffic.md
+TRAFFIC_PROFILE = "profiles/skinny_gemv_cfg2_m16_hbm_traffic.md"
+
+
+def profile_traffic_bytes():
+  """HBM bytes per launch of the decode GEMV kernel as the rocprofv3 counter summary under profiles/ states it
+  (the figure in bold there: scaled FETCH_SIZE + WRITE_SIZE), or None when the file or the figure is missing."""
+  import re
+  try:
+    text = open(os.path.join(ROOT, TRAFFIC_PROFILE)).read()
+  except OSError:
+    return None
+  m = re.search(r"\*\*([0-9.]+) MB\*\*", text)
+  return float(m.group(1)) * 1e6 if m else None
 
 
 def gemv_bytes(m, n, k, w_bytes_per_elem=1.0, x_b=2, s_b=2, out_b=2, n_scale_rows=1, zp=False):
@@ -346,8 +358,8 @@ def main():
           "frac": round(achieved / HBM_PEAK_GBPS, 4),
           # HBM bytes per launch measured with rocprofv3 (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from an
           # elementwise kernel of known size); it is a profile result, not re-measured by this script
-          "traffic": TRAFFIC_BYTES_PER_LAUNCH,
-          "traffic_source": "profiles/skinny_gemv_cfg2_m16_hbm_traffic.md",
+          "traffic": profile_traffic_bytes(),
+          "traffic_source": TRAFFIC_PROFILE,
           "kernel": "qmm_skinny_kernel<bf16, int8, MT=1> (4 computing + 4 copying waves)",
           "avg_launch_us": round(ev_ms * 1e3, 3),
       },
@@ -380,6 +392,14 @@ def main():
     for w in wv:
       qmm.invalidate_weight_cache(w)  # frees the tiled copies too
     del wv, sv, w
+
+    # config 1: fp32 activations, 1 MB of weights (latency-bound: reported only)
+    x1, w1, s1 = [t.to(dev) for t in cases.uniform_int8(8, 1024, 1024, torch.float32, torch.float32, seed=1)]
+    _, ev, _ = time_calls([lambda: op(x1, w1, s1)], steps2, 12, use_graph)
+    b1 = gemv_bytes(8, 1024, 1024, x_b=4, s_b=4, out_b=4)
+    extra["cfg1_fp32_M8_1024x1024"] = {"us": round(ev * 1e3, 3), "GBps": round(b1 / ev / 1e6, 1),
+                                       "frac_hbm": round(b1 / ev / 1e6 / HBM_PEAK_GBPS, 4),
+                                       "note": "1.1 MB per call: launch latency, not bandwidth"}
 
     # blockwise int4 (config 3)
     x3, w3, s3, z3, _ = cases.blockwise(16, 4096, 4096, 128, 4, torch.bfloat16, symmetric=False, seed=4)
@@ -471,9 +491,11 @@ def main():
           op(x_in[w.shape[1]], w, s, quantize_activation=qa)
 
       _, ev, _ = time_calls([run_layer], 20, 5, use_graph)
-      extra[f"llama3_8b_layer_linears_{tag}"] = {"us": round(ev * 1e3, 2),
-                                                 "note": "us: one set of weights (218 MB), cache-warm between iterations; "
-                                                         "us_cold: three sets in turn"}
+      extra[f"llama3_8b_layer_linears_{tag}"] = {
+          "us_one_weight_set": round(ev * 1e3, 2),
+          "note": "us_one_weight_set: the same 218 MB of weights every iteration (they do not stay in the 256 MB Infinity "
+                  "Cache next to the activations and outputs: close to cold); us_cold: three sets in turn; per_linear: "
+                  "each projection alone over the three sets in turn (cold), with its share of the roofline that bounds it"}
 
       def run_set(ls):
         for name, (w, s) in ls.items():
@@ -481,6 +503,16 @@ def main():
 
       _, ev, _ = time_calls([(lambda ls=ls: run_set(ls)) for ls in sets_s], 21, 6, use_graph)
       extra[f"llama3_8b_layer_linears_{tag}"]["us_cold"] = round(ev * 1e3, 2)
+      per = {}
+      for name in ("q", "k", "o", "gate", "down"):  # (v is k's shape, up is gate's)
+        n_, k_ = shapes[name]
+        _, ev1, _ = time_calls([(lambda ls=ls: op(x_in[k_], ls[name][0], ls[name][1], quantize_activation=qa)) for ls in sets_s],
+                               21, 6, use_graph)
+        if qa:
+          per[name] = {"us": round(ev1 * 1e3, 2), "frac_mfma": round(2.0 * m * n_ * k_ / ev1 / 1e9 / INT8_PEAK_TOPS, 4)}
+        else:
+          per[name] = {"us": round(ev1 * 1e3, 2), "frac_hbm": round(gemv_bytes(m, n_, k_) / ev1 / 1e6 / HBM_PEAK_GBPS, 4)}
+      extra[f"llama3_8b_layer_linears_{tag}"]["per_linear"] = per
 
       # the same layer with q/k/v and gate/up concatenated along N: 4 launches instead of 7
       def cat(names):
@@ -535,48 +567,69 @@ def main():
     cores = os.cpu_count() or 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
-    oracle.quantized_matmul(x16, w_cpu, s_cpu)  # warm-up
-    t_runs = []
-    t_start = time.perf_counter()
-    while len(t_runs) < 5 or (time.perf_counter() - t_start < 10.0 and len(t_runs) < 50):
-      t0 = time.perf_counter()
-      oracle.quantized_matmul(x16, w_cpu, s_cpu)
-      t_runs.append(time.perf_counter() - t0)
-    t_med = sorted(t_runs)[len(t_runs) // 2]
-    # the other configurations' CPU figures (bounded samples), next to their GPU entries
-    if extra:
-      def cpu_time(fn, budget_s=4.0, max_runs=20):
+
+    def cpu_time(fn, budget_s, max_runs=50, min_runs=5):
+      """(min, median, runs) of the wall time of fn over at least min_runs calls (one untimed call first)."""
+      fn()
+      runs, t_begin = [], time.perf_counter()
+      while len(runs) < min_runs or (time.perf_counter() - t_begin < budget_s and len(runs) < max_runs):
+        t0 = time.perf_counter()
         fn()
-        runs, t_begin = [], time.perf_counter()
-        while len(runs) < 3 or (time.perf_counter() - t_begin < budget_s and len(runs) < max_runs):
-          t0 = time.perf_counter()
-          fn()
-          runs.append(time.perf_counter() - t0)
-        return sorted(runs)[len(runs) // 2], len(runs)
+        runs.append(time.perf_counter() - t0)
+      runs.sort()
+      return runs[0], runs[len(runs) // 2], len(runs)
+
+    def cpu_entry(t_min, t_med, n, amount, unit, scale, what):
+      return {"value": round(amount / t_med / scale, 4), "value_best_run": round(amount / t_min / scale, 4), "unit": unit,
+              "cores": cores, "kind": "port", "runs": n, "ms_median": round(t_med * 1e3, 2), "ms_min": round(t_min * 1e3, 2),
+              "sample": what}
+
+    t_min, t_med, n_runs = cpu_time(lambda: oracle.quantized_matmul(x16, w_cpu, s_cpu), 8.0)
+    result["cpu_baseline"] = cpu_entry(
+        t_min, t_med, n_runs, bytes16, "GB/s", 1e9,
+        f"{n_runs} full calls of the same M=16 workload through the CPU oracle (torch {torch.__version__} eager ops, the "
+        f"reference's CPU-tensor semantics); value from the median, value_best_run from the fastest call")
+    # the other configurations (bounded samples), next to their GPU entries where there is one
+    if extra:
+      per_config = {}
+      x1, w1, s1 = cases.uniform_int8(8, 1024, 1024, torch.float32, torch.float32, seed=1)[:3]
+      t = cpu_time(lambda: oracle.quantized_matmul(x1, w1, s1), 1.0)
+      per_config["cfg1_fp32_8x1024x1024"] = cpu_entry(*t, gemv_bytes(8, 1024, 1024, x_b=4, s_b=4, out_b=4), "GB/s", 1e9,
+                                                      "full calls of config 1")
+      for m in (1, 4):
+        xm = x16[:m].contiguous()
+        t = cpu_time(lambda: oracle.quantized_matmul(xm, w_cpu, s_cpu), 2.0)
+        per_config[f"cfg2_decode_gemv_M{m}"] = cpu_entry(*t, gemv_bytes(m, N_OUT, K_IN), "GB/s", 1e9, f"full calls of config 2, M={m}")
+      per_config["cfg2_decode_gemv_M16"] = result["cpu_baseline"]
       x3, w3, s3, z3, _ = cases.blockwise(16, 4096, 4096, 128, 4, torch.bfloat16, symmetric=False, seed=4)
-      t3, n3 = cpu_time(lambda: oracle.quantized_matmul(x3, w3, s3, z3, block_size=128, int4_weight=True))
+      t = cpu_time(lambda: oracle.quantized_matmul(x3, w3, s3, z3, block_size=128, int4_weight=True), 3.0)
+      b3 = gemv_bytes(16, 4096, 4096, 0.5, n_scale_rows=32, zp=True)
+      per_config["cfg3_blockwise_int4_M16"] = cpu_entry(*t, b3, "GB/s", 1e9, "full calls of config 3 (algorithmic bytes of the packed int4 weight)")
       if "blockwise_int4_M16" in extra:
-        extra["blockwise_int4_M16"]["cpu_baseline"] = {
-            "value": round(extra["blockwise_int4_M16"]["algorithmic_bytes"] / t3 / 1e9, 3), "unit": "GB/s", "cores": cores,
-            "kind": "port", "sample": f"median of {n3} full calls of the same workload through the CPU oracle; {t3 * 1e3:.1f} ms per call"}
+        extra["blockwise_int4_M16"]["cpu_baseline"] = per_config["cfg3_blockwise_int4_M16"]
       rows4 = 128  # of the 2048 rows: the CPU's int32 matmul takes seconds for all of them
       x4c = cases.outlier_activations(2048, K_IN, torch.bfloat16, seed=1234)[:rows4].contiguous()
       s4c = s_cpu.float()
-      t4, n4 = cpu_time(lambda: oracle.quantized_matmul(x4c, w_cpu, s4c, quantize_activation=True), budget_s=8.0, max_runs=10)
+      t = cpu_time(lambda: oracle.quantized_matmul(x4c, w_cpu, s4c, quantize_activation=True), 6.0, max_runs=10)
+      per_config["cfg4_w8a8_prefill"] = cpu_entry(
+          *t, 2.0 * rows4 * N_OUT * K_IN, "TOP/s", 1e12,
+          f"calls on the first {rows4} of the 2048 rows (quantize + int32 matmul + scales) through the CPU oracle")
       if "w8a8_prefill_M2048" in extra:
-        extra["w8a8_prefill_M2048"]["cpu_baseline"] = {
-            "value": round(2.0 * rows4 * N_OUT * K_IN / t4 / 1e12, 4), "unit": "TOP/s", "cores": cores, "kind": "port",
-            "sample": f"median of {n4} calls on the first {rows4} of the 2048 rows (quantize + int32 matmul + scales) "
-                      f"through the CPU oracle; {t4 * 1e3:.0f} ms per call"}
-    result["cpu_baseline"] = {
-        "value": round(bytes16 / t_med / 1e9, 3),
-        "unit": "GB/s",
-        "cores": cores,
-        "kind": "port",
-        "sample": f"median of {len(t_runs)} full calls of the same M=16 workload through the CPU oracle "
-                  f"(torch {torch.__version__} eager ops, the reference's CPU-tensor semantics); "
-                  f"{t_med * 1e3:.1f} ms per call",
-    }
+        extra["w8a8_prefill_M2048"]["cpu_baseline"] = per_config["cfg4_w8a8_prefill"]
+      # config 5, decode step: the seven linears at M = 32 (218 MB of int8 weights converted to bf16 per call)
+      g5c = cases.gen(5)
+      shapes5 = [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096), (4096, 14336)]
+      lin5 = [(torch.randint(-127, 128, (n, k), generator=g5c, dtype=torch.int32).to(torch.int8),
+               (torch.rand(n, generator=g5c) * 0.01).bfloat16(), torch.randn(32, k, generator=g5c).bfloat16()) for n, k in shapes5]
+
+      def layer_cpu():
+        for w_, s_, x_ in lin5:
+          oracle.quantized_matmul(x_, w_, s_)
+
+      t = cpu_time(layer_cpu, 4.0, max_runs=10)
+      bytes5 = sum(gemv_bytes(32, n, k) for n, k in shapes5)
+      per_config["cfg5_layer_decode_M32"] = cpu_entry(*t, bytes5, "GB/s", 1e9, "the seven linears of config 5 at M=32, one after the other")
+      extra["cpu_baseline_per_config"] = per_config
   print(json.dumps(result))
 
 

@@ -38,7 +38,9 @@ constexpr size_t kScratchBytes = kScratchXq + 2 * round_up((size_t)kScratchRows 
 
 }  // namespace
 
-static __device__ __align__(256) unsigned char qmm_noalloc_scratch[kScratchBytes];
+// (`used`: no device code names the array - kernels get its address as an argument - so nothing else keeps
+// it in the code object)
+static __device__ __align__(256) __attribute__((used)) unsigned char qmm_noalloc_scratch[kScratchBytes];
 
 namespace {
 
@@ -46,22 +48,26 @@ namespace {
 // host-side handle: the address comes from hipGetSymbolAddress, once per device, with that
 // device current, and is what kernels, memsets and copies must be given.
 std::mutex g_scratch_mu;
-void* g_scratch_ptr[64] = {};
+std::atomic<void*> g_scratch_ptr[64] = {};
 
 int scratch_of_current_device(void** out) {
   int dev = -1;
   int rc = qmm_check_hip(hipGetDevice(&dev), "w8a8_linear_noalloc hipGetDevice");
   if (rc != XLA_AMD_QMM_OK) return rc;
   if (dev < 0 || dev >= 64) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "w8a8_linear_noalloc: device ordinal %d out of range", dev);
-  std::lock_guard<std::mutex> lock(g_scratch_mu);
-  if (!g_scratch_ptr[dev]) {
-    void* p = nullptr;
-    rc = qmm_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(qmm_noalloc_scratch)), "w8a8_linear_noalloc hipGetSymbolAddress");
-    if (rc != XLA_AMD_QMM_OK) return rc;
-    if (!p) return qmm_fail(XLA_AMD_QMM_EHIP, "w8a8_linear_noalloc: hipGetSymbolAddress returned a null address");
-    g_scratch_ptr[dev] = p;
+  // (the steady state is one atomic load; the lock is only taken while a device's address is still unknown)
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (!p) {
+      rc = qmm_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(qmm_noalloc_scratch)), "w8a8_linear_noalloc hipGetSymbolAddress");
+      if (rc != XLA_AMD_QMM_OK) return rc;
+      if (!p) return qmm_fail(XLA_AMD_QMM_EHIP, "w8a8_linear_noalloc: hipGetSymbolAddress returned a null address");
+      g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
   }
-  *out = g_scratch_ptr[dev];
+  *out = p;
   return XLA_AMD_QMM_OK;
 }
 
