@@ -477,6 +477,24 @@ def test_narrow_channel_groups_parity(ops, n, m, zp):
   check(got, expected, f"n={n} m={m} zp={zp}")
 
 
+@pytest.mark.parametrize("n,k", [(36864, 1024), (33002, 512), (40000, 4096), (128256, 512)])
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("zp", [False, True])
+def test_streaming_kernel_with_resident_x(ops, n, k, m, zp):
+  """More channel groups than wave slots and up to 16 rows: persistent waves that each stream a run of groups,
+  x resident in LDS (one and two copy chunks of x, group widths 10 / 16, a channel count that is not a multiple
+  of the group), against the oracle."""
+  x, w, s, _ = cases.per_channel_int8(m, n, k, torch.bfloat16, torch.bfloat16, seed=n + m)
+  z = (torch.randn(n, generator=cases.gen(3)) * 0.01).to(torch.bfloat16) if zp else None
+  expected = oracle.quantized_matmul(x, w, s, z)
+  got = torch.ops.xla.quantized_matmul(*dev(x, w, s, z))
+  check(got, expected, f"n={n} k={k} m={m} zp={zp}")
+  if m == 16 and not zp:
+    x16 = x.half()
+    got16 = torch.ops.xla.quantized_matmul(*dev(x16, w, s.half()))
+    check(got16, oracle.quantized_matmul(x16, w, s.half()), f"f16 n={n} k={k}")
+
+
 def test_w8a8_tiles_and_tails(ops):
   # every workgroup tile the kernel offers, on shapes with M/N/K tails
   for bm, bn in ((32, 32), (64, 32), (64, 64), (128, 128), (128, 256), (256, 256)):

@@ -27,6 +27,8 @@ SOURCES = [
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=1"], "qmm_skinny_bf16.o"),
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=2"], "qmm_skinny_f16.o"),
     ("qmm_skinny.hip", ["-DQMM_SKINNY_XT=0"], "qmm_skinny_f32.o"),
+    ("qmm_skinny_resident.hip", ["-DQMM_SKINNY_XT=1"], "qmm_skinny_resident_bf16.o"),
+    ("qmm_skinny_resident.hip", ["-DQMM_SKINNY_XT=2"], "qmm_skinny_resident_f16.o"),
     ("qmm_wo_gemm.hip", ["-DQMM_WO_XT=1", "-DQMM_WO_MT=4"], "qmm_wo_gemm_bf16_mt4.o"),
     ("qmm_wo_gemm.hip", ["-DQMM_WO_XT=2", "-DQMM_WO_MT=4"], "qmm_wo_gemm_f16_mt4.o"),
     ("qmm_wo_gemm_bw.hip", ["-DQMM_WO_BW_XT=1"], "qmm_wo_gemm_bw_bf16.o"),

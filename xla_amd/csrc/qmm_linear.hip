@@ -38,9 +38,11 @@ constexpr size_t kScratchBytes = kScratchXq + 2 * round_up((size_t)kScratchRows 
 
 }  // namespace
 
-// (`used`: no device code names the array - kernels get its address as an argument - so nothing else keeps
-// it in the code object)
-static __device__ __align__(256) __attribute__((used)) unsigned char qmm_noalloc_scratch[kScratchBytes];
+// (No device code names the array - kernels get its address as an argument.  What keeps it in the code object
+// is the host's reference through HIP_SYMBOL below: the compiler emits a static device variable that host code
+// names under a symbol the runtime can look up.  Marking it `used` instead breaks that: the library then aborts
+// inside hipGetSymbolAddress.)
+static __device__ __align__(256) unsigned char qmm_noalloc_scratch[kScratchBytes];
 
 namespace {
 

@@ -36,3 +36,9 @@ int qmm_skinny_launch_f16(const SkinnyArgs& a, int bits, bool haszp, hipStream_t
 // K slices the streaming kernel should run a per-channel launch of M <= 32 rows in (1 = none):
 // few output channels against a long K, where every workgroup would otherwise copy all of x.
 int qmm_skinny_k_slices(int64_t M, int64_t N, int64_t K, int64_t C, int bits, int* k_per_slice);
+
+// The persistent form of the streaming kernel with all of x resident in LDS (qmm_skinny_resident.hip): how many
+// workgroups a launch would run with (0: not a launch for it), and its launchers.
+int qmm_skinny_resident_workgroups(const SkinnyArgs& a, int x_dt, int bits);
+int qmm_skinny_resident_launch_bf16(const SkinnyArgs& a, bool haszp, int workgroups, hipStream_t stream);
+int qmm_skinny_resident_launch_f16(const SkinnyArgs& a, bool haszp, int workgroups, hipStream_t stream);

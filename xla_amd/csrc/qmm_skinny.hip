@@ -842,6 +842,15 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
   // registers of the int8 per-channel kernels with one dtype throughout.  Measured with cold
   // weights: 28672 x 4096 at M = 32 29.0 -> 25.9 us, at M = 16 24.8 -> 23.5; 18432 x 8192 at
   // M = 1 37.4 -> 28.6 us (288 workgroups had been a round and an eighth).
+  // More channel groups than wave slots, up to 16 rows of x that fit in LDS whole: persistent waves that each
+  // stream a run of groups without a break (qmm_skinny_resident.hip).  Measured with cold weights at M = 16 / M = 1:
+  // see the numbers at that kernel's dispatch in the design notes.
+  if constexpr (BITS == 8 && XT != XLA_AMD_DT_F32 && MT == 1) {
+    if (const int wgs = qmm_skinny_resident_workgroups(a, XT, BITS)) {
+      if constexpr (XT == XLA_AMD_DT_BF16) return qmm_skinny_resident_launch_bf16(a, haszp, wgs, stream);
+      else return qmm_skinny_resident_launch_f16(a, haszp, wgs, stream);
+    }
+  }
   if constexpr (BITS == 8 && XT != XLA_AMD_DT_F32) {
     const bool uni = a.scale_dt == XT && a.zp_dt == XT && a.out_dt == XT && a.dot_dt == XT && a.store_dt == XT;
     if (kw == 1 && perch && uni && workgroups(1) > kComputeUnits)
