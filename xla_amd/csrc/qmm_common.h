@@ -60,6 +60,13 @@ __device__ __forceinline__ void qmm_lds_barrier() {
 // s_barrier.  For code that keeps global -> LDS copies in flight across the barrier and does
 // its own vmcnt waits (a workgroup-scope fence makes the compiler wait for every such copy,
 // since they are LDS writes); the memory clobber keeps LDS accesses on their side of it.
+// Waits until at most N of this wave's vector memory operations are outstanding (they complete in order);
+// the other counters are left alone.
+template <int N> __device__ __forceinline__ void qmm_wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
 __device__ __forceinline__ void qmm_bare_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }

@@ -36,6 +36,15 @@ __device__ __forceinline__ i32x4 cvt_w8(uint32_t d0, uint32_t d1) {
   return o;
 }
 
+// Two int8 weights (the low or the high half of a dword) -> two elements of the x dtype: a quarter of cvt_w8.
+template <int XT, class HiC>
+__device__ __forceinline__ uint32_t cvt_w2(uint32_t d, HiC) {
+  constexpr int sh = HiC::value ? 16 : 0;
+  const float lo = (float)(int8_t)(d >> sh), hi = (float)(int8_t)(d >> (sh + 8));
+  if constexpr (XT == XLA_AMD_DT_BF16) return pack_hi16(lo, hi);
+  else return pack_f16(lo, hi);
+}
+
 // 8 packed int4 weights (one dword, nibble j = column P[j], biased by 8) -> 8
 // elements (1 + u/16) of the x dtype, u = w + 8 in 0..15.  The caller undoes
 // the affine map with the exact x sum: sum w*x = 16*(sum a*x - 1.5*sum x).

@@ -72,16 +72,17 @@ using namespace qmm_frag;
 
 template <int MT, int NG> struct WoCfg {
   static constexpr int BM = 16 * MT;
-  static constexpr int X_TILE = BM * 256;                      // bytes of the x columns of one step (128 columns, 2-byte x)
-  // Weight blocks in flight per wave and channel group (register ring): two for the 64-row tile
-  // with two channel groups per wave, whose short steps (16 MFMAs per half block) would otherwise
-  // wait for memory every time and which has the registers; one for the others (four channel
-  // groups or 128 rows: the accumulators leave no room for a second block, and their steps are long).
-  static constexpr int P = (MT < 8 && NG == 2) ? 2 : 1;
-  static constexpr int kFit = kLds / (2 * X_TILE) / P * P;     // steps per chunk slot that fit twice (whole trips around the ring)
-  static constexpr int CS = kFit < 8 ? kFit : 8;               // steps per chunk
-  static_assert(CS >= P, "two chunk slots must fit in LDS");
-  static constexpr int lds_bytes(int steps) { return (steps <= CS ? steps : 2 * CS) * X_TILE; }
+  static constexpr int X_TILE = BM * 256;  // bytes of the x columns of one step (128 columns, 2-byte x)
+  // Half blocks of weights (64 columns) in flight per wave and channel group: a ring of registers.  A half is
+  // requested again as soon as it has been used, so it has (H - 1) / 2 steps to arrive.  The 128 x 256 tile
+  // (128 accumulator registers) has room for three; the others hold five: their steps are short.
+  static constexpr int H = (MT == 8 && NG == 4) ? 3 : 5;
+  static_assert(H % 2 == 1, "a step uses two halves: an odd ring visits every phase in H steps");
+  // x tiles (one step each) in LDS: a ring that the copying waves fill R - 1 tiles ahead of the computing waves
+  static constexpr int kFit = kLds / X_TILE;
+  static constexpr int R = kFit < 8 ? kFit : 8;
+  static_assert(R >= 3, "the x ring needs room to run ahead");
+  static constexpr int lds_bytes(int steps) { return (steps < R ? steps : R) * X_TILE; }
 };
 
 // The dtypes of the epilogue: those of the call, or (UNI) all equal to x's dtype and known at
@@ -180,18 +181,18 @@ __device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, in
 
 // One unit of work: a tile of rows x channels over one K slice.
 struct WoItem {
-  int m0, g0, ks, k_begin, steps, n_chunks, rows;  // g0: first channel group of the column tile
+  int m0, g0, ks, k_begin, steps, rows;  // g0: first channel group of the column tile
 };
 
 // The kernel is persistent: workgroup b takes the work items b, b + gridDim.x, ... one after the
-// other.  The chunk ring simply runs on across items, so the copying waves fetch the first
-// chunk of the next item while the computing waves finish and store the current one, and the
+// other.  The ring of x tiles simply runs on across items, so the copying waves fetch the first
+// tiles of the next item while the computing waves finish and store the current one, and the
 // computing waves request the next item's first weights before they store.
 template <int XT, int MT, int NG, bool HASZP, bool UNI>
 __global__ void __launch_bounds__((kComputeWaves + kCopyWaves) * 64)
 qmm_wo_gemm_kernel(WoGemmArgs a) {
   using Cfg = WoCfg<MT, NG>;
-  constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE, CS = Cfg::CS;
+  constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE;
   constexpr int GPT = 4 * NG;  // channel groups per workgroup: NG per computing wave (groups of a.G channels, 16 or fewer)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -213,46 +214,50 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     w.g0 = (tile % tiles_n) * GPT;
     w.k_begin = w.ks * a.k_per_split;
     w.steps = (min(K, w.k_begin + a.k_per_split) - w.k_begin) / 128;  // >= 1
-    w.n_chunks = (w.steps + CS - 1) / CS;
     w.rows = min(BM, M - w.m0);  // live rows of this tile
     return w;
   };
 
   if (__builtin_expect(wave >= kComputeWaves, 0)) {
-    // ---- copying waves: chunk after chunk of x into the two slots in turn, rows shared among them ----
+    // ---- copying waves: the x tiles of this workgroup's steps, one after the other (across items), into
+    // the slots of the ring in turn; tile t lives in slot t % R.  D = R - 1 tiles are requested ahead: the
+    // loads of a wave return in order, so tile n is there once no more than the loads of the D - 1 tiles
+    // after it are in flight, whatever the memory latency (up to D - 1 steps of it are hidden).
     const int cw = wave - kComputeWaves;
-    auto chunk_load = [&](const WoItem& w, int c, int slot_i) __attribute__((always_inline)) {
-      const int s0 = c * CS;
-      const int nst = min(CS, w.steps - s0);
-      char* const slot = smem + slot_i * (CS * X_TILE);
-      const char* const xb = (const char*)a.x + ((size_t)w.m0 * K + w.k_begin) * 2;
-      // a row of one step is 256 bytes: an instruction copies four consecutive rows
-      // (lane l: row l/16 of the four, chunk l%16), swizzled on the source side
-      for (int r4 = cw * 4; r4 < w.rows; r4 += kCopyWaves * 4) {
-        const int row = min(r4 + (lane >> 4), w.rows - 1);  // rows past the end repeat the last one
+    constexpr int R = Cfg::R, D = R - 1;
+    constexpr int L = BM / (4 * kCopyWaves);  // loads per tile and wave: an instruction copies four rows of 256 bytes
+    static_assert((D - 1) * L < 64, "the loads in flight must fit the counter");
+    int total = 0;  // steps of this workgroup
+    for (int i = blockIdx.x; i < n_items; i += gridDim.x) total += item_of(i).steps;
+    int q_it = blockIdx.x, q_s = 0, issued = 0;  // the next tile to request: step q_s of item q_it
+    WoItem q = item_of(q_it);
+    auto issue = [&]() __attribute__((always_inline)) {
+      if (issued >= total) return;
+      char* const dst = smem + (issued % R) * X_TILE;
+      const char* const xb = (const char*)a.x + ((size_t)q.m0 * K + q.k_begin) * 2 + (size_t)q_s * 256;
+#pragma unroll
+      for (int i = 0; i < L; ++i) {
+        // (lane l: row l / 16 of the four, 16-byte chunk l % 16, swizzled on the source side;
+        // rows past the end repeat the last one)
+        const int r4 = (cw + i * kCopyWaves) * 4;
+        const int row = min(r4 + (lane >> 4), q.rows - 1);
         const int chunk = (lane & 15) ^ (row & 15);
-        const char* src = xb + (size_t)row * ((size_t)K * 2) + (size_t)s0 * 256 + chunk * 16;
-        char* dst = slot + r4 * 256;
-        for (int t = 0; t < nst; ++t)
-          __builtin_amdgcn_global_load_lds((const void*)(src + t * 256), (lds_ptr_t)(dst + t * X_TILE), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const void*)(xb + (size_t)row * ((size_t)K * 2) + chunk * 16),
+                                         (lds_ptr_t)(dst + r4 * 256), 16, 0, 0);
+      }
+      ++issued;
+      if (++q_s == q.steps) {
+        q_s = 0;
+        q_it += gridDim.x;
+        if (q_it < n_items) q = item_of(q_it);
       }
     };
-    int it = blockIdx.x;
-    WoItem cur = item_of(it);
-    int c = 0, ring = 0;  // ring: chunks since the kernel began; chunk `ring` lives in slot ring % 2
-    chunk_load(cur, 0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    for (;;) {
-      qmm_bare_barrier();  // chunk `ring` is there, chunk ring - 1 has been read
-      ++c; ++ring;
-      if (c == cur.n_chunks) {
-        it += gridDim.x;
-        if (it >= n_items) break;
-        cur = item_of(it);
-        c = 0;
-      }
-      chunk_load(cur, c, ring & 1);
-      __builtin_amdgcn_s_waitcnt(0x0F70);
+    for (int d = 0; d < D; ++d) issue();
+    for (int n = 0; n < total; ++n) {
+      if (issued - n == D) qmm_wait_vmcnt<(D - 1) * L>();  // the tiles n + 1 .. n + D - 1 may be in flight
+      else qmm_wait_vmcnt<0>();                             // (the first and the last tiles of the workgroup)
+      qmm_bare_barrier();  // tile n is there; the computing waves have read tile n - 1
+      issue();             // tile n + D into the slot of tile n - 1
     }
     return;
   }
@@ -263,73 +268,81 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   // the group's last row again and their results are dropped.
   const int n_blk = K / 128;  // blocks per channel group in the tiled weight
   const int blk_bytes = G * 128, half_bytes = G * 64;
-  constexpr int P = Cfg::P;
-  const uint8_t* wp[NG];
-  i32x4 wreg[P][NG][2];  // ring slot s % P holds the block of step s
+  constexpr int H = Cfg::H, R = Cfg::R;
+  const uint8_t* wp[NG];  // wave-uniform: the first half block of the item for each channel group (scalar registers)
+  const uint32_t w_lane = (uint32_t)((g * G + min(r, G - 1)) * 16);  // this lane's 16 bytes inside a half block
+  i32x4 wreg[H][NG];  // ring: half q of the item (block q / 2, columns 64 (q % 2) ..) lives in slot q % H
   auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
       const int grp_u = w.g0 + wave * NG + gi;
       const int grp = min(grp_u, groups - 1);  // groups past N re-read the last one
-      wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * blk_bytes + (g * G + min(r, G - 1)) * 16;
+      wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * blk_bytes;
     });
   };
-  auto load_half = [&](int blk, auto slotc, auto hc) __attribute__((always_inline)) {
-    constexpr int slot = slotc, h = hc;
+  // half q of the item into its slot (a half past the end is the last one again: never used, and no branch
+  // around the loads: the counts of loads in flight stay known at compile time on every path)
+  auto request = [&](int q, int last, auto slotc) __attribute__((always_inline)) {
+    constexpr int slot = slotc;
+    const int qq = min(q, last);
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      wreg[slot][gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * blk_bytes + h * half_bytes));
+      const uint8_t* half = wp[gi] + (size_t)qq * half_bytes;  // uniform: scalar base + lane offset
+      wreg[slot][gi] = __builtin_nontemporal_load((const i32x4*)(half + (size_t)w_lane));
     });
   };
-  // the first P blocks of an item (a block past the end of a short item is the last one again: never used)
   auto load_first = [&](const WoItem& w) __attribute__((always_inline)) {
-    qmm_static_for<P>([&](auto pc) {
-      constexpr int slot = pc;
-      const int blk = min(slot, w.steps - 1);
-      load_half(blk, qmm_const<slot>{}, qmm_const<0>{});
-      load_half(blk, qmm_const<slot>{}, qmm_const<1>{});
-    });
+    qmm_static_for<H>([&](auto hc) { request((int)hc, 2 * w.steps - 1, hc); });
   };
 
   f32x4 acc[NG][MT], xs[MT];
-  // one step (128 columns) out of LDS tile `tile` with the weights of ring slot SLOT; with
-  // REFILL the slot's registers are refilled with block `next` as soon as each half has been used
-  auto compute = [&](int tile, int next, auto slotc, auto refillc) __attribute__((always_inline)) {
-    constexpr int slot = slotc;
-    constexpr bool kRefill = refillc != 0;
-    const char* xbase = smem + tile * X_TILE;
-    qmm_static_for<4>([&](auto jc) {
-      constexpr int j = jc;
-      i32x4 xq[MT];
+  // One step (128 columns): step s of an item of S steps, x out of LDS slot `xslot`, weights out of the ring
+  // slots PH (columns 0 .. 63) and PH + 1 (columns 64 .. 127); each slot is requested again (half + H of the
+  // item) as soon as it has been used.
+  // The step is software-pipelined by hand over its 4 * NG weight fragments (fragment f = j * NG + gi: columns
+  // 32 g + 8 j .. of channel group gi).  Between the MT MFMAs of fragment f sit the conversions of fragment f + 1
+  // (a quarter of them, three instructions, after every MT / 4 th MFMA: about what fits in the issue slots that an
+  // MFMA leaves free), and in the last group of a j every MFMA is followed by the LDS read that replaces its x
+  // fragment with that of j + 1.  A scheduling fence after each such unit keeps the order: left to itself the
+  // compiler emits the conversions and the MFMAs of a fragment as two separate runs, the matrix pipe idles during
+  // the conversions, and with one computing wave per SIMD nothing else fills the gap.
+  auto compute = [&](int xslot, int s, int S, auto phc) __attribute__((always_inline)) {
+    constexpr int PH = phc;
+    const char* xrow = smem + xslot * X_TILE + r * 256;  // this lane's row of each 16-row tile
+    const int last = 2 * S - 1;
+    auto xfrag = [&](int j, int mt) __attribute__((always_inline)) {
+      return *(const i32x4*)(xrow + mt * (16 * 256) + (((4 * g + j) ^ r) * 16));
+    };
+    i32x4 xq[MT];
+    qmm_static_for<MT>([&](auto mc) { xq[(int)mc] = xfrag(0, mc); });
+    i32x4 af;
+    {
+      const i32x4 src = wreg[PH][0];
+      af = cvt_w8<XT>((uint32_t)src[0], (uint32_t)src[1]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    constexpr int kEvery = MT / 4;  // a quarter of the next fragment after every kEvery th MFMA
+    qmm_static_for<4 * NG>([&](auto fc) {
+      constexpr int f = fc, j = f / NG, gi = f % NG;
+      constexpr bool kLastGroup = gi == NG - 1, kMore = f + 1 < 4 * NG;
+      constexpr int jn = kMore ? (f + 1) / NG : 0, gn = kMore ? (f + 1) % NG : 0;
+      i32x4 af_next = af;
       qmm_static_for<MT>([&](auto mc) {
         constexpr int mt = mc;
-        xq[mt] = *(const i32x4*)(xbase + (16 * mt + r) * 256 + (((4 * g + j) ^ r) * 16));
+        acc[gi][mt] = mfma16<XT>(af, xq[mt], acc[gi][mt]);
+        if constexpr (HASZP && kLastGroup) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt], xs[mt]);
+        if constexpr (kMore && mt % kEvery == 0) {
+          constexpr int q = mt / kEvery;  // element q of the fragment: bytes 2 (q & 1), 2 (q & 1) + 1 of dword q / 2
+          af_next[q] = (int)cvt_w2<XT>((uint32_t)wreg[(PH + (jn >> 1)) % H][gn][(jn & 1) * 2 + q / 2], qmm_const<(q & 1)>{});
+        }
+        if constexpr (kLastGroup && j + 1 < 4) xq[mt] = xfrag(j + 1, mt);
+        __builtin_amdgcn_sched_barrier(0);
       });
-      qmm_static_for<NG>([&](auto gc) {
-        constexpr int gi = gc;
-        const i32x4 src = wreg[slot][gi][j >> 1];
-        const i32x4 af = cvt_w8<XT>((uint32_t)src[(j & 1) * 2], (uint32_t)src[(j & 1) * 2 + 1]);
-        qmm_static_for<MT>([&](auto mc) {
-          constexpr int mt = mc;
-          acc[gi][mt] = mfma16<XT>(af, xq[mt], acc[gi][mt]);
-        });
-      });
-      if constexpr (HASZP) {
-        qmm_static_for<MT>([&](auto mc) {
-          constexpr int mt = mc;
-          xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt], xs[mt]);
-        });
+      if constexpr (kLastGroup && (j & 1)) {
+        request(2 * s + (j >> 1) + H, last, qmm_const<(PH + (j >> 1)) % H>{});
+        __builtin_amdgcn_sched_barrier(0);
       }
-      if constexpr (kRefill && (j & 1)) load_half(next, qmm_const<slot>{}, qmm_const<(j >> 1)>{});
-    });
-  };
-  // P consecutive steps starting at step s (s % P == 0) of which `live` exist; NREF of them refill
-  // their slot (the refills are compile-time so that the loads in flight stay countable)
-  auto compute_group = [&](int tile, int s, int live, auto nrefc) __attribute__((always_inline)) {
-    constexpr int nref = nrefc;
-    qmm_static_for<P>([&](auto pc) {
-      constexpr int slot = pc;
-      if (slot == 0 || slot < live) compute(tile + slot, s + slot + P, qmm_const<slot>{}, qmm_const<(slot < nref ? 1 : 0)>{});
+      af = af_next;
     });
   };
 
@@ -337,33 +350,27 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   WoItem cur = item_of(it);
   set_weights(cur);
   load_first(cur);
-  int ring = 0;
+  int xslot = 0;  // LDS slot of the next x tile: the tiles of all items of the workgroup follow each other round the ring
+  auto step = [&](int s, int S, auto phc) __attribute__((always_inline)) {
+    qmm_bare_barrier();  // the tile is there (the copying waves waited for it); the tile before it has been read
+    compute(xslot, s, S, phc);
+    xslot = xslot + 1 == R ? 0 : xslot + 1;
+  };
   for (;;) {
     qmm_static_for<MT>([&](auto mc) {
       constexpr int mt = mc;
       xs[mt] = f32x4{0, 0, 0, 0};
       qmm_static_for<NG>([&](auto gc) { acc[(int)gc][mt] = f32x4{0, 0, 0, 0}; });
     });
+    // H steps visit the H phases of the weight ring (step s starts at half 2 s, slot 2 s % H): unrolled, so that
+    // every register of the ring is named at compile time; the last S % H steps follow one by one
+    const int S = cur.steps;
     int s = 0;
-    for (int c = 0; c < cur.n_chunks; ++c, ++ring) {
-      qmm_bare_barrier();  // chunk `ring` is there (the copying waves waited for it)
-      const int tile0 = (ring & 1) * CS - c * CS;
-      if constexpr (P == 1) {
-        int s_end = min(cur.steps, (c + 1) * CS);
-        if (c + 1 == cur.n_chunks) --s_end;  // the item's last step fetches nothing more: it runs after the loop
-        for (; s < s_end; ++s) compute(tile0 + s, s + 1, qmm_const<0>{}, qmm_const<1>{});
-        if (c + 1 == cur.n_chunks) compute(tile0 + s, 0, qmm_const<0>{}, qmm_const<0>{});
-      } else {
-        const int s_end = min(cur.steps, (c + 1) * CS);
-        // groups of P steps (a chunk holds whole groups); the item's last P steps fetch nothing more
-        for (; s < s_end; s += P) {
-          const int left = cur.steps - s;
-          if (left >= 2 * P) compute_group(tile0 + s, s, P, qmm_const<P>{});
-          else if (left == 3) compute_group(tile0 + s, s, 2, qmm_const<1>{});
-          else compute_group(tile0 + s, s, left, qmm_const<0>{});
-        }
-      }
-    }
+    for (; s + H <= S; s += H)
+      qmm_static_for<H>([&](auto kc) { step(s + (int)kc, S, qmm_const<(2 * (int)kc) % H>{}); });
+    qmm_static_for<H - 1>([&](auto kc) {
+      if (s + (int)kc < S) step(s + (int)kc, S, qmm_const<(2 * (int)kc) % H>{});
+    });
 
     // the next item's first weights are requested before this item's results are stored: a wait
     // for them then does not include the stores
@@ -493,9 +500,11 @@ int launch(const WoGemmArgs& a, hipStream_t stream) {
   // one dtype throughout (x, scale, zero point, dot, out, store): the epilogue's dtypes fold at compile time
   const bool uni = a.scale_dt == XT && a.zp_dt == XT && a.dot_dt == XT && a.out_dt == XT && a.store_dt == XT;
   if constexpr (MT == 8 && NG == 4) {
-    // (the 128 x 256 tile with the row sums of x does not fit the register file: the plan never asks for it)
+    // (the 128 x 256 tile fits the register file neither with the row sums of x nor with dtypes known only at run
+    // time: the plan never asks for the first, and the second takes the 128 x 128 tile)
     if (a.zp) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: no 128 x 256 tile with a zero point");
-    return uni ? go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, false>);
+    if (!uni) return launch<XT, MT, 2>(a, stream);
+    return go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>);
   } else {
     if (uni) return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, true>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, true>);
     return a.zp ? go(qmm_wo_gemm_kernel<XT, MT, NG, true, false>) : go(qmm_wo_gemm_kernel<XT, MT, NG, false, false>);
