@@ -9,15 +9,17 @@
 // over workgroups (each then copies only its slice of x); the partial sums of a split
 // go to a workspace and a second kernel adds them in a fixed order and finishes them.
 //
-// Operands.  Weights come from the tiled copy (xla_amd_qmm_tile_weight): one 2 KB block per
-// 16 channels x 128 columns, already in MFMA operand order, so a wave loads its fragments
-// straight into registers: no LDS traffic and no transposition for weights.  x goes through
-// LDS: the workgroup's rows, a chunk of K steps (128 columns each) at a time, in two chunk
-// slots; four extra waves do nothing but copy the next chunk (global -> LDS without
-// registers) while the four computing waves use the current one, and the workgroup meets
-// once per chunk.  (The computing waves must not issue such copies themselves: with copies
-// in flight the compiler can no longer count their register loads in flight and turns every
-// wait of the loop into a wait for all of them.)
+// Operands.  Weights come from the tiled copy (xla_amd_qmm_tile_weight): per group of G <= 16 channels and 128
+// columns one block, already in MFMA operand order, so a wave loads its fragments straight into registers: no
+// LDS traffic and no transposition for weights.  An MFMA row set is 16 consecutive channels whatever G is
+// (channel n = row n % G of group n / G; every lane keeps the offset of its row, the base is scalar), so the
+// kernel wastes no MFMA rows on groups narrower than 16.  Per row set a wave keeps a ring of three or five half
+// blocks (64 columns) in registers and asks for a half again as soon as it has been used.
+// x goes through LDS: the workgroup's rows, one step (128 columns) per tile, in a ring of 5 (128 rows) or 8
+// (64 rows) tiles; four extra waves do nothing but copy (global -> LDS without registers) up to R - 1 tiles
+// ahead of the four computing waves, and the workgroup meets once per step.  (The computing waves must not issue
+// such copies themselves: with copies in flight the compiler can no longer count their register loads in flight
+// and turns every wait of the loop into a wait for all of them.)
 //
 // MFMA mapping (v_mfma_f32_16x16x32_bf16/f16, A = weights, B = x^T), as in the streaming
 // kernel: lane l is (r = l%16, g = l/16); for a block of 128 columns the lane supplies, for
@@ -70,14 +72,17 @@ constexpr int kLds = 160 * 1024;
 
 using namespace qmm_frag;
 
+// Half blocks of weights (64 columns) in flight per wave and MFMA row set: a ring of registers.  A half is
+// requested again as soon as it has been used, so it has (H - 1) / 2 steps to arrive.  The 128 x 256 tile
+// (128 accumulator registers) has room for three, and so has the 64 x 256 tile with a zero point and dtypes
+// known only at run time; the others hold five: their steps are short.
+template <int MT, int NG, bool HASZP, bool UNI> constexpr int wo_ring_halves() {
+  return ((MT == 8 && NG == 4) || (MT == 4 && NG == 4 && HASZP && !UNI)) ? 3 : 5;
+}
+
 template <int MT, int NG> struct WoCfg {
   static constexpr int BM = 16 * MT;
   static constexpr int X_TILE = BM * 256;  // bytes of the x columns of one step (128 columns, 2-byte x)
-  // Half blocks of weights (64 columns) in flight per wave and channel group: a ring of registers.  A half is
-  // requested again as soon as it has been used, so it has (H - 1) / 2 steps to arrive.  The 128 x 256 tile
-  // (128 accumulator registers) has room for three; the others hold five: their steps are short.
-  static constexpr int H = (MT == 8 && NG == 4) ? 3 : 5;
-  static_assert(H % 2 == 1, "a step uses two halves: an odd ring visits every phase in H steps");
   // x tiles (one step each) in LDS: a ring that the copying waves fill R - 1 tiles ahead of the computing waves
   static constexpr int kFit = kLds / X_TILE;
   static constexpr int R = kFit < 8 ? kFit : 8;
@@ -140,8 +145,7 @@ __device__ __forceinline__ void wo_store4(void* out, int m, int n, int N, const 
 }
 
 // Stores the first cnt (1 .. 4) of four consecutive channels of row m starting at channel n, n even: in
-// pairs where the row length allows it (channel groups narrower than 16 start on even, not on
-// four-aligned channels, and their last lane holds two channels).
+// pairs where the row length allows it (rows whose length is no multiple of 4).
 __device__ __forceinline__ void wo_store_some(void* out, int m, int n, int N, int cnt, const float o[4], int store_dt) {
   const size_t idx = (size_t)m * N + n;
   if ((N & 1) == 0) {
@@ -181,7 +185,7 @@ __device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, in
 
 // One unit of work: a tile of rows x channels over one K slice.
 struct WoItem {
-  int m0, g0, ks, k_begin, steps, rows;  // g0: first channel group of the column tile
+  int m0, n0, ks, k_begin, steps, rows;  // n0: first channel of the column tile
 };
 
 // The kernel is persistent: workgroup b takes the work items b, b + gridDim.x, ... one after the
@@ -193,7 +197,7 @@ __global__ void __launch_bounds__((kComputeWaves + kCopyWaves) * 64)
 qmm_wo_gemm_kernel(WoGemmArgs a) {
   using Cfg = WoCfg<MT, NG>;
   constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE;
-  constexpr int GPT = 4 * NG;  // channel groups per workgroup: NG per computing wave (groups of a.G channels, 16 or fewer)
+  constexpr int BN = 64 * NG;  // channels per workgroup: NG MFMA row sets of 16 per computing wave
   extern __shared__ __attribute__((aligned(16))) char smem[];
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -201,8 +205,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, g = lane >> 4;
   const int M = a.M, N = a.N, K = a.K, G = a.G;
-  const int groups = (N + G - 1) / G;
-  const int tiles_n = (groups + GPT - 1) / GPT;
+  const int tiles_n = (N + BN - 1) / BN;
   const int tiles = tiles_n * ((M + BM - 1) / BM);
   const int n_items = tiles * a.split;
   // item -> (K slice, row tile, column tile), column tiles fastest: workgroups that run together share x rows
@@ -211,7 +214,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     const int tile = it % tiles;
     w.ks = it / tiles;
     w.m0 = (tile / tiles_n) * BM;
-    w.g0 = (tile % tiles_n) * GPT;
+    w.n0 = (tile % tiles_n) * BN;
     w.k_begin = w.ks * a.k_per_split;
     w.steps = (min(K, w.k_begin + a.k_per_split) - w.k_begin) / 128;  // >= 1
     w.rows = min(BM, M - w.m0);  // live rows of this tile
@@ -263,21 +266,25 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   }
 
   // ---- computing waves ----
-  // wave w owns the channel groups g0 + w*NG .. + NG-1 of the item's column tile.  Group p holds the
-  // channels G p .. G p + G - 1 in MFMA rows 0 .. G - 1; the rows from G on (groups narrower than 16) read
-  // the group's last row again and their results are dropped.
+  // wave w owns the channels n0 + 64 w .. + 63 of the item's column tile as NG MFMA row sets of 16 consecutive
+  // channels, whatever the width G of the channel groups of the tiled weight: channel n lies in group n / G at
+  // row n % G, so the 16 rows of a set come out of one or two groups and every lane keeps its own offset
+  // (channels past N read the last one again; their results are dropped).
   const int n_blk = K / 128;  // blocks per channel group in the tiled weight
   const int blk_bytes = G * 128, half_bytes = G * 64;
-  constexpr int H = Cfg::H, R = Cfg::R;
-  const uint8_t* wp[NG];  // wave-uniform: the first half block of the item for each channel group (scalar registers)
-  const uint32_t w_lane = (uint32_t)((g * G + min(r, G - 1)) * 16);  // this lane's 16 bytes inside a half block
-  i32x4 wreg[H][NG];  // ring: half q of the item (block q / 2, columns 64 (q % 2) ..) lives in slot q % H
+  constexpr int H = wo_ring_halves<MT, NG, HASZP, UNI>(), R = Cfg::R;
+  static_assert(H % 2 == 1, "a step uses two halves: an odd ring visits every phase in H steps");
+  const uint8_t* wp;     // wave-uniform: the first half block of the item in the tile's first channel group
+  uint32_t w_lane[NG];   // from there to this lane's 16 bytes of row set gi (less than 2^32: 270 channels of K columns)
+  i32x4 wreg[H][NG];     // ring: half q of the item (block q / 2, columns 64 (q % 2) ..) lives in slot q % H
   auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
+    const int p0 = w.n0 / G;
+    wp = a.w + ((size_t)p0 * n_blk + w.k_begin / 128) * blk_bytes;
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      const int grp_u = w.g0 + wave * NG + gi;
-      const int grp = min(grp_u, groups - 1);  // groups past N re-read the last one
-      wp[gi] = a.w + ((size_t)grp * n_blk + w.k_begin / 128) * blk_bytes;
+      const int ch = min(w.n0 + (wave * NG + gi) * 16 + r, N - 1);
+      const int p = ch / G, row = ch - p * G;
+      w_lane[gi] = (uint32_t)(p - p0) * ((uint32_t)n_blk * (uint32_t)blk_bytes) + (uint32_t)((g * G + row) * 16);
     });
   };
   // half q of the item into its slot (a half past the end is the last one again: never used, and no branch
@@ -287,8 +294,8 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     const int qq = min(q, last);
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      const uint8_t* half = wp[gi] + (size_t)qq * half_bytes;  // uniform: scalar base + lane offset
-      wreg[slot][gi] = __builtin_nontemporal_load((const i32x4*)(half + (size_t)w_lane));
+      const uint8_t* half = wp + (size_t)qq * half_bytes;  // uniform: scalar base + lane offset
+      wreg[slot][gi] = __builtin_nontemporal_load((const i32x4*)(half + (size_t)w_lane[gi]));
     });
   };
   auto load_first = [&](const WoItem& w) __attribute__((always_inline)) {
@@ -386,12 +393,12 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
 
     // ---- results: four consecutive channels of one row per lane ----
     const int m0 = done.m0;
-    // channels of this lane for group gi of its wave: n .. n + cnt - 1 (cnt <= 4; computed where they are
-    // used: the 128 x 256 tile has no register to keep them in)
-    const int g_first = done.g0 + wave * NG;
+    // channels of this lane for row set gi of its wave: n .. n + cnt - 1, n a multiple of 4 (cnt <= 4, or <= 0 past N;
+    // computed where they are used: the 128 x 256 tile has no register to keep them in)
+    const int n_first = done.n0 + wave * (NG * 16) + 4 * g;
     auto chan = [&](int gi, int& n, int& cnt) __attribute__((always_inline)) {
-      n = (g_first + gi) * G + 4 * g;
-      cnt = min(min(G - 4 * g, N - n), 4);
+      n = n_first + gi * 16;
+      cnt = min(N - n, 4);
     };
     if (a.split == 1) {
       const WoDts<XT, UNI> dts(a);
@@ -417,7 +424,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
             int n, cnt;
             chan(gi, n, cnt);
             if (m < M && cnt > 0) {
-              if (kVec && cnt == 4 && (n & 3) == 0) {  // four channels, four-aligned: one store
+              if (kVec && cnt == 4) {  // four channels (n is a multiple of 4): one store
                 if constexpr (kVec && UNI && !HASZP && XT == XLA_AMD_DT_BF16) {
                   wo_finish_store_bf16(a.out, m, n, N, sraw[gi], acc[gi][mt]);
                 } else {
@@ -454,7 +461,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       });
       if constexpr (HASZP) {
         // partial row sums of x: once per row tile and K slice (the first column tile's first wave, channel lanes 0..15)
-        if (done.g0 == 0 && wave == 0 && g == 0) {
+        if (done.n0 == 0 && wave == 0 && g == 0) {
           qmm_static_for<MT>([&](auto mc) {
             constexpr int mt = mc;
             const int m = m0 + 16 * mt + r;
@@ -483,8 +490,7 @@ int cu_count() {
 template <int XT, int MT, int NG>
 int launch(const WoGemmArgs& a, hipStream_t stream) {
   using Cfg = WoCfg<MT, NG>;
-  const int64_t groups = ((int64_t)a.N + a.G - 1) / a.G;
-  const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * ((groups + 4 * NG - 1) / (4 * NG)) * a.split;
+  const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * (((int64_t)a.N + 64 * NG - 1) / (64 * NG)) * a.split;
   const int steps = a.k_per_split / 128;
   // one workgroup per compute unit (its LDS and registers leave room for no second one); each walks its share of the items
   const int cus = cu_count();
@@ -618,8 +624,7 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
   p.mt = M <= 64 ? 4 : 8;
   const int64_t bm = 16 * p.mt;
   const int64_t tiles_m = (M + bm - 1) / bm;
-  const int64_t g_ch = xla_amd_qmm_tile_group(N, K, K, 8);
-  const int64_t groups = (N + g_ch - 1) / g_ch;  // a column tile is 4 * ng channel groups
+  const int64_t groups = (N + 15) / 16;  // MFMA row sets of 16 channels: a column tile is 4 * ng of them
   p.ng = 4;
   if ((tiles_m * ((groups + 15) / 16) < 192 && N > 128) || (has_zp && p.mt == 8)) p.ng = 2;
   const int64_t tiles = tiles_m * ((groups + 4 * p.ng - 1) / (4 * p.ng));
@@ -675,7 +680,7 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
     return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm: dot dtype must be x's or f32");
   if (x_dt == XLA_AMD_DT_F32) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x must be bf16 or f16");
   if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: K=%lld must be a multiple of 128", (long long)K);
-  if (N > (1 << 30) || K > (1 << 24) || M > (1 << 24))
+  if (N > (1 << 30) || K > (1 << 23) || M > (1 << 24))
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: dimension too large");
   if (((uintptr_t)x | (uintptr_t)w_tiled) & 15)
     return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm: x and w must be 16-byte aligned");
