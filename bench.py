@@ -189,6 +189,9 @@ def main():
   ap.add_argument("--no-graph", action="store_true", help="time eager calls instead of a HIP graph replay")
   ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+  ap.add_argument("--no-sclk", action="store_true",
+                  help="do not sample the shader clock (it starts rocm-smi as a child process, which a counter-collecting "
+                       "profiler run must not do)")
   ap.add_argument("--timeline", action="store_true",
                   help="instead of the benchmark: in-kernel timeline of the decode GEMV (diagnostic build of the "
                        "streaming kernel, libxla_amd_qmm_timeline.so); prints a table, not the JSON line")
@@ -276,6 +279,8 @@ def main():
     import subprocess
     import threading
     found = []
+    if args.no_sclk:
+      return None
 
     def sample():
       time.sleep(seconds * 0.4)
@@ -459,11 +464,15 @@ def main():
     s2 = s_cpu.to(dev)
     x4b = torch.randn(m4, K_IN, generator=cases.gen(2)).bfloat16().to(dev)  # config 2's activations: N(0, 1)
     _, ev_wo, _ = time_calls([lambda: op(x4b, w0, s2)], steps4, 5, use_graph)
+    sclk_wo = observed_sclk_mhz(lambda: op(x4b, w0, s2))
+    _, ev_wo_sustained, _ = time_calls([lambda: op(x4b, w0, s2)], 4 * steps4, 5, use_graph)
     extra["weight_only_prefill_M2048"] = {
         "us": round(ev_wo * 1e3, 2),
+        "us_sustained": round(ev_wo_sustained * 1e3, 2),
+        "sclk_mhz_observed": sclk_wo,
         "roofline": {"bound": "mfma", "achieved": round(ops4 / ev_wo / 1e9, 1), "peak": BF16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(ops4 / ev_wo / 1e9 / BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "qmm_wo_gemm_kernel<bf16, 128 x 256 tile>"},
+                     "kernel": "qmm_wo_gemm_kernel<bf16, 128 x 256 tile> (persistent, 4 computing + 4 copying waves)"},
         "vs_w8a8_end_to_end": round(ev_wo / ev_e2e, 2),
     }
     del x4, x4b, xq, xsc

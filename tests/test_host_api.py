@@ -357,3 +357,16 @@ def test_no_kernel_of_the_built_library_spills_registers():
   kernels = json.load(open(build.RESOURCES_PATH))
   assert len(kernels) > 50
   assert [k for k in kernels if k.get("scratch_bytes_per_lane", 0) > 0] == []
+
+
+def test_headline_kernels_keep_their_code_budget():
+  """The build records every kernel's code bytes; the decode kernels, whose cold prologue is part of every launch, have a budget."""
+  import json
+  from xla_amd import build
+  if not os.path.exists(build.RESOURCES_PATH):
+    pytest.skip("library not built by xla_amd.build in this tree")
+  by_name = {k["kernel"]: k for k in json.load(open(build.RESOURCES_PATH))}
+  assert all("code_bytes" in k and k["code_bytes"] > 0 for k in by_name.values())
+  for name, budget in build.CODE_BUDGET_BYTES.items():
+    assert name in by_name, name
+    assert by_name[name]["code_bytes"] <= budget, (name, by_name[name]["code_bytes"], budget)

@@ -95,6 +95,38 @@ def _kernel_resources(report: str, unit: str):
   return kernels
 
 
+# Code bytes per kernel, read from the symbol table of the device code object inside each object file of this
+# build.  A launch starts with a cold instruction cache, and the decode kernels run their straight-line prologue
+# once: every instruction on the way to the first load is a few nanoseconds of a launch that lasts about twelve
+# microseconds, so the two headline kernels have a budget, and the build fails when one of them outgrows it.
+LLVM_BIN = os.environ.get("LLVM_BIN", "/opt/rocm/llvm/bin")
+CODE_BUDGET_BYTES = {
+    # mangled name of the kernel: bytes (decode GEMV, bf16 / int8 per channel, 16 rows at most; its persistent form)
+    "_ZN12_GLOBAL__N_117qmm_skinny_kernelILi1ELi8ELi1ELi1ELi1ELb0ELb1ELi4ELi512EEEv10SkinnyArgs": 8192,
+    "_ZN12_GLOBAL__N_126qmm_skinny_resident_kernelILi1ELb0EEEv10SkinnyArgs": 11264,
+}
+
+
+def _code_bytes(obj: str):
+  """{kernel symbol: bytes} of the gfx950 code object bundled in `obj`."""
+  fat, dev = obj + ".fatbin", obj + ".gfx950.co"
+  try:
+    _run(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", obj, fat])
+    _run([os.path.join(LLVM_BIN, "clang-offload-bundler"), "--type=o", "--targets=hipv4-amdgcn-amd-amdhsa--gfx950",
+          "--input=" + fat, "--output=" + dev, "--unbundle"])
+    table = _run([os.path.join(LLVM_BIN, "llvm-readelf"), "-sW", dev])
+  finally:
+    for f in (fat, dev):
+      if os.path.exists(f):
+        os.remove(f)
+  sizes = {}
+  for line in table.splitlines():
+    f = line.split()
+    if len(f) >= 8 and f[3] == "FUNC" and f[6] != "UND":
+      sizes[f[7]] = int(f[2])
+  return sizes
+
+
 def build(verbose: bool = False, jobs: int = 8) -> str:
   os.makedirs(OBJ_DIR, exist_ok=True)
   objs = []
@@ -105,6 +137,10 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     out = _run([HIPCC] + FLAGS + ["-Rpass-analysis=kernel-resource-usage"] + extra +
                ["-c", os.path.join(CSRC, src), "-o", obj])
     kernels = _kernel_resources(out, name)
+    sizes = _code_bytes(obj) if kernels else {}  # (a unit without kernels carries no device code object)
+    for k in kernels:
+      if k["kernel"] in sizes:
+        k["code_bytes"] = sizes[k["kernel"]]
     if verbose:
       # (a remark is followed by the source line it points at and a caret line)
       rest = "\n".join(l for l in out.splitlines() if "kernel-resource-usage" not in l and
@@ -126,6 +162,16 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     raise RuntimeError("kernels with a scratch frame (register spills):\n" +
                        "\n".join("  %s: %s (%d bytes per lane, %d VGPRs)" % (k["unit"], k["kernel"], k["scratch_bytes_per_lane"],
                                                                             k.get("vgprs", -1)) for k in spilling))
+  by_name = {k["kernel"]: k for k in kernels}
+  over = []
+  for name, budget in CODE_BUDGET_BYTES.items():
+    k = by_name.get(name)
+    if k is None or "code_bytes" not in k:
+      raise RuntimeError("kernel with a code budget is not in the build (renamed?): " + name)
+    if k["code_bytes"] > budget:
+      over.append("  %s: %d bytes of code, budget %d" % (name, k["code_bytes"], budget))
+  if over:
+    raise RuntimeError("kernels over their code budget:\n" + "\n".join(over))
   tmp = LIB_PATH + ".tmp"
   _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", "-o", tmp] + objs)
   os.replace(tmp, LIB_PATH)
