@@ -56,8 +56,9 @@ def gemv_bytes(m, n, k, w_bytes_per_elem=1.0, x_b=2, s_b=2, out_b=2, n_scale_row
   return int(n * k * w_bytes_per_elem + m * k * x_b + scale_bytes + m * n * out_b)
 
 
-def timeline(torch, _lib, qmm, cases, dev, m, hot):
-  """In-kernel timeline of the decode GEMV (x bf16 [m,4096], w int8 [14336,4096]).
+def timeline(torch, _lib, qmm, cases, dev, m, hot, config=2):
+  """In-kernel timeline of the decode GEMV (x bf16 [m,4096], w int8 [14336,4096]), or with config=3 of the
+  blockwise int4 + zero point matmul (x bf16 [m,4096], w int4 [32,128,4096]).
 
   The diagnostic build of the streaming kernel notes, per wave, the chip-wide 100 MHz
   counter at fixed points (entry, first weights requested / landed, first x chunk in
@@ -71,25 +72,39 @@ def timeline(torch, _lib, qmm, cases, dev, m, hot):
   raw = ctypes.CDLL(_lib.lib_path())
   raw.xla_amd_qmm_timeline_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
   raw.xla_amd_qmm_timeline_read.restype = ctypes.c_int
-  x, w_cpu, s_cpu, _ = cases.per_channel_int8(m, N_OUT, K_IN, torch.bfloat16, torch.bfloat16, seed=2)
-  x, s_d, w0 = x.to(dev), s_cpu.to(dev), w_cpu.to(dev)
-  wt0 = qmm._tiled_weight(w0, 8, _lib.W_NK)
-  n_rot = 1 if hot else 12
-  wts = [wt0] + [wt0.clone() for _ in range(n_rot - 1)]
-  out = torch.empty(m, N_OUT, dtype=torch.bfloat16, device=dev)
-  bf = _lib.DT_BF16
+  if config == 3:
+    n_out, k_in, row_bytes = 4096, 4096, 2048
+    x, w3, s3, z3, _ = cases.blockwise(m, n_out, k_in, 128, 4, torch.bfloat16, symmetric=False, seed=4)
+    x, s_d, z_d = x.to(dev), s3.to(dev), z3.to(dev)
+    n_rot = 1 if hot else 40  # 40 x 8.4 MB: more than the Infinity Cache
+    wts = [w3.to(dev) for _ in range(n_rot)]
+    op = torch.ops.xla.quantized_matmul
+    what = f"blockwise int4 + zero point x bf16 [{m},{k_in}] x w int4 [{k_in // 128},128,{n_out}]"
 
-  def run(wt):
-    _lib.check(lib.xla_amd_qmm_weight_only_skinny(x.data_ptr(), wt.data_ptr(), s_d.data_ptr(), None, out.data_ptr(), m,
-                                                  N_OUT, K_IN, K_IN, 8, bf, bf, bf, bf, bf, bf,
-                                                  torch.cuda.current_stream().cuda_stream), "weight_only_skinny")
+    def run(wt):
+      op(x, wt, s_d, z_d, block_size=128, int4_weight=True)
+  else:
+    n_out, k_in, row_bytes = N_OUT, K_IN, K_IN
+    x, w_cpu, s_cpu, _ = cases.per_channel_int8(m, N_OUT, K_IN, torch.bfloat16, torch.bfloat16, seed=2)
+    x, s_d, w0 = x.to(dev), s_cpu.to(dev), w_cpu.to(dev)
+    wt0 = qmm._tiled_weight(w0, 8, _lib.W_NK)
+    n_rot = 1 if hot else 12
+    wts = [wt0] + [wt0.clone() for _ in range(n_rot - 1)]
+    out = torch.empty(m, N_OUT, dtype=torch.bfloat16, device=dev)
+    bf = _lib.DT_BF16
+    what = f"decode GEMV x bf16 [{m},{K_IN}] x w int8 [{N_OUT},{K_IN}]"
+
+    def run(wt):
+      _lib.check(lib.xla_amd_qmm_weight_only_skinny(x.data_ptr(), wt.data_ptr(), s_d.data_ptr(), None, out.data_ptr(), m,
+                                                    N_OUT, K_IN, K_IN, 8, bf, bf, bf, bf, bf, bf,
+                                                    torch.cuda.current_stream().cuda_stream), "weight_only_skinny")
 
   for wt in wts:
     run(wt)
   torch.cuda.synchronize()
   g = torch.cuda.CUDAGraph()
   with torch.cuda.graph(g):
-    for i in range(24):
+    for i in range(max(24, n_rot)):
       run(wts[i % n_rot])
   t_pre = time.perf_counter()
   while (time.perf_counter() - t_pre) * 1e3 < PREWARM_MS:
@@ -105,7 +120,7 @@ def timeline(torch, _lib, qmm, cases, dev, m, hot):
   ncomp = nwv - 4  # the last four waves of a workgroup copy x
   t0 = t[:, :, 0][live].min()
   rel = np.where(t > 0, (t - t0) * 0.01, np.nan)  # 100 MHz ticks -> us since the first wave's entry
-  print(f"decode GEMV x bf16 [{m},{K_IN}] x w int8 [{N_OUT},{K_IN}], {'one weight copy (cache-resident)' if hot else '12 rotating weight copies (cold)'}: "
+  print(f"{what}, {'one weight copy (cache-resident)' if hot else f'{n_rot} rotating weight copies (cold)'}: "
         f"{nb} workgroups x ({ncomp} computing + {nwv - ncomp} copying waves)")
 
   def table(title, waves, names):
@@ -116,7 +131,7 @@ def timeline(torch, _lib, qmm, cases, dev, m, hot):
       if v.size:
         print(f"  {name:34s} {v.min():7.2f} {np.median(v):7.2f} {v.max():7.2f}")
 
-  n_steps = K_IN // 512
+  n_steps = row_bytes // 512
   table("computing waves", slice(0, ncomp),
         [(0, "entry"), (1, "first weights requested"), (2, "first weights landed"), (3, "first x chunk in LDS (met)")] +
         [(4 + i, f"step {i} done") for i in range(min(n_steps - 1, 22))] +
@@ -200,6 +215,8 @@ def main():
                        "launch shapes (diagnostic library); prints a table")
   ap.add_argument("--timeline-hot", action="store_true", help="with --timeline: one weight copy (cache-resident) instead of rotating ones")
   ap.add_argument("--timeline-m", type=int, default=16, help="with --timeline: rows of x")
+  ap.add_argument("--timeline-config", type=int, default=2, choices=(2, 3),
+                  help="with --timeline: 2 = decode GEMV (int8 per channel), 3 = blockwise int4 + zero point 4096 x 4096")
   ap.add_argument("--calibrate-copy", action="store_true",
                   help="also run a plain 256 MiB device copy (known traffic, for scaling rocprof byte counters)")
   args = ap.parse_args()
@@ -305,7 +322,7 @@ def main():
   use_graph = not args.no_graph
 
   if args.timeline:
-    timeline(torch, _lib, qmm, cases, dev, args.timeline_m, args.timeline_hot)
+    timeline(torch, _lib, qmm, cases, dev, args.timeline_m, args.timeline_hot, args.timeline_config)
     return
   if args.stream_probe:
     stream_probe(torch, _lib, dev)
