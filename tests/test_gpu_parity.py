@@ -137,6 +137,20 @@ def test_blockwise_shapes(ops, xdt, bits):
     check(out, exp, f"blockwise {m,n,k,c}")
 
 
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("sym", [False, True])
+def test_blockwise_int4_eight_wave_k_split(ops, xdt, sym):
+  """Packed int4, K = 4096, at most 256 channel groups, up to 16 rows: eight computing waves split K
+  (256 weight bytes per row and step); block sizes that divide the 512 columns of a step."""
+  for (m, n, c) in [(16, 4096, 128), (1, 4096, 256), (7, 1000, 512), (16, 24, 128), (3, 4080, 128)]:
+    x, w, s, z, _ = cases.blockwise(m, n, 4096, c, 4, xdt, symmetric=sym, seed=100 + m)
+    exp = oracle.quantized_matmul(x, w, s, z, block_size=c, int4_weight=True)
+    before = ops.counters["skinny_mfma"]
+    out = torch.ops.xla.quantized_matmul(*dev(x, w, s, z), block_size=c, int4_weight=True)
+    check(out, exp, f"blockwise int4 {m,n,c}")
+    assert ops.counters["skinny_mfma"] == before + 1
+
+
 def test_int4_per_channel(ops):
   g = cases.gen(9)
   x = torch.randn(7, 512, generator=g).bfloat16()

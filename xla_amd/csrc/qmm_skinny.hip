@@ -124,7 +124,7 @@ struct SkinnyCfg {
     const int x = tiles * X_TILE;
     return x > kRedBytes ? x : kRedBytes;
   }
-  static_assert(WSEG == 512 || (WSEG == 256 && BITS == 8), "weight segment");
+  static_assert(WSEG == 512 || WSEG == 256, "weight segment");
 };
 
 // Extra waves per workgroup that do nothing but copy x (and the blockwise scales) into LDS (see the
@@ -856,6 +856,17 @@ int launch_split(const SkinnyArgs& a, bool haszp, hipStream_t stream) {
     if (kw == 1 && perch && uni && workgroups(1) > kComputeUnits)
       return haszp ? launch_kernel<XT, BITS, MT, 1, kRedRaw, true, true, 8, kWSeg>(a, stream)
                    : launch_kernel<XT, BITS, MT, 1, kRedRaw, false, true, 8, kWSeg>(a, stream);
+  }
+  // Blockwise int4 against few channels (one channel group per compute unit at most) with all of x in one chunk:
+  // a wave's step is issue-bound arithmetic (every block has its own rounding sequence), so eight computing waves
+  // with half-length steps (256 weight bytes per row) split K eight ways.
+  if constexpr (BITS == 4 && XT != XLA_AMD_DT_F32 && MT == 1) {
+    using Cfg8 = SkinnyCfg<XT, BITS, MT, 8, 8, 256>;
+    const int steps8 = (a.k_per_slice + Cfg8::KS - 1) / Cfg8::KS;
+    if (!perch && Cfg8::KS % a.C == 0 && a.k_per_slice % Cfg8::KS == 0 && groups * a.slices <= kComputeUnits &&
+        steps8 == 8 && Cfg8::kFits)
+      return haszp ? launch_kernel<XT, BITS, MT, 8, kRedScaled, true, true, 8, 256>(a, stream)
+                   : launch_kernel<XT, BITS, MT, 8, kRedScaled, false, true, 8, 256>(a, stream);
   }
   if (kw == 1) {
     return perch ? launch_zp<XT, BITS, MT, 1, kRedRaw>(a, haszp, stream)
