@@ -143,6 +143,8 @@ def test_config4_quantized_matmul_int8_bf16_out_full(ops):
 # ---- the float branch of the dedicated kernel (f32 accumulation, f32 scale, one cast) --------------------
 @pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16, torch.float32])
 def test_dedicated_kernel_float_branch(ops, xdt):
+  """Self-consistency (kernel against this build's oracle), not reference parity: no test of the reference runs the
+  float branch, and that each block's dot product stays in f32 there is an assumption."""
   from xla_amd.experimental.hip_kernels.quantized_matmul_kernel import quantized_matmul_int8 as kernel
   for (m, n, k) in [(16, 14336, 4096), (5, 256, 1024), (40, 100, 384), (3, 8, 5)]:
     x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + n)

@@ -170,3 +170,15 @@ def test_blockwise_k_slices(ops, xdt):
     assert ops.counters["wo_gemm"] == before + 1
     rl2 = check(out, exp, f"blockwise K slices {m, n, k, c, bits, asym, xdt}")
     assert rl2 < 1e-3, (m, n, k, c, bits, rl2)
+
+
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+def test_wo_gemm_several_rounds_of_tiles(ops, xdt):
+  """More 128 x 256 tiles than compute units, the last round part full: persistent workgroups walk two items or
+  one (also: a last column tile narrower than 256, rows whose count is no multiple of 16 or of 128)."""
+  for (m, n, k) in [(1056, 7680, 256), (1100, 7500, 384), (2048, 14336, 128)]:
+    assert -(-m // 128) * -(-n // 256) > 256
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m)
+    exp = oracle.quantized_matmul(x, w, s)
+    out = wo_gemm(ops, x.cuda(), w.cuda(), s.cuda(), None)
+    check(out, exp, f"several rounds {m,n,k}")
