@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define XLA_AMD_QMM_ABI_VERSION 4
+#define XLA_AMD_QMM_ABI_VERSION 5
 
 /* return codes */
 #define XLA_AMD_QMM_OK 0
@@ -209,6 +209,25 @@ int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, const void*
                                  void* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
                                  int64_t K, int64_t C, int bits, int x_dt, int scale_dt, int zp_dt, int dot_dt,
                                  int out_dt, int store_dt, void* stream);
+
+/*
+ * The same for f32 activations (xla_amd_qmm_dispatch sends 128 rows or more
+ * here; fewer take the streaming kernel, 16 rows per pass): out f32 [M,N] = F.linear(x, w) * scaler
+ * (- rowsum(x) (x) zp), xla_quantized_matmul.py:113-114 with x of any floating
+ * dtype, here f32.  x is split into three bf16 parts whose sum is x to the last
+ * bit (hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid)) and the bf16
+ * GEMM runs over the 3 K columns of the parts against the weight three times
+ * over, accumulating in f32: every product is exact, so the result differs from
+ * an f32 dot product by the order of the additions only.  Per-channel int8
+ * weights, K % 128 == 0, 3 K <= 2^23; scale / zp of any floating dtype.
+ * `workspace`: xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(M, N, K) bytes
+ * of device memory (the three parts: 6 M K), 16-byte aligned, free again when
+ * the call's work has completed.
+ */
+size_t xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int xla_amd_qmm_weight_only_gemm_f32(const float* x, const void* w_tiled, const void* scale, const void* zp,
+                                     float* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                                     int64_t K, int scale_dt, int zp_dt, void* stream);
 
 /*
  * Weight-only quantized matmul for any shape, reading the operator's own

@@ -182,3 +182,19 @@ def test_wo_gemm_several_rounds_of_tiles(ops, xdt):
     exp = oracle.quantized_matmul(x, w, s)
     out = wo_gemm(ops, x.cuda(), w.cuda(), s.cuda(), None)
     check(out, exp, f"several rounds {m,n,k}")
+
+
+@pytest.mark.parametrize("sdt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("zp", [False, True])
+def test_f32_rows_through_the_tiled_gemm(ops, sdt, zp):
+  """128 rows of f32 x or more: split into three bf16 parts (exact), bf16 MFMA GEMM with f32 accumulation; against
+  the f32 oracle to summation-order accuracy (the tolerance of the f32 streaming kernel's test)."""
+  for (m, n, k) in [(128, 64, 128), (300, 700, 1024), (130, 4096, 2048), (1000, 520, 384)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, torch.float32, sdt, seed=m)
+    z = (torch.randn(n, generator=cases.gen(m + 1)) * 0.5).to(sdt) if zp else None
+    exp = oracle.quantized_matmul(x, w, s, z)
+    before = ops.counters["wo_gemm"]
+    out = torch.ops.xla.quantized_matmul(x.cuda(), w.cuda(), s.cuda(), None if z is None else z.cuda())
+    assert ops.counters["wo_gemm"] == before + 1, "f32 rows did not take the tiled GEMM"
+    rl2 = check(out, exp, f"f32 rows {m,n,k,sdt,zp}")
+    assert rl2 < 1e-5, rl2

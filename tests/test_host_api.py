@@ -35,7 +35,7 @@ def test_library_exports_every_declared_symbol():
   for n in names:
     assert hasattr(lib, n), f"{n} declared in the header but not exported"
   assert sorted(_lib.SIGNATURES) == names, "ctypes signatures out of sync with the header"
-  assert lib.xla_amd_qmm_abi_version() == 4
+  assert lib.xla_amd_qmm_abi_version() == 5
 
 
 def test_header_cites_reference_for_each_entry_point():
@@ -56,7 +56,12 @@ def test_dispatcher_regimes():
   # channels and a long K (the streaming kernel over K slices, behind the same entry point with a workspace)
   assert d(33, 14336, 4096, 4096, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
   assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
-  assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F32, 0) == _lib.KERNEL_SKINNY_MFMA
+  assert d(2048, 14336, 4096, 4096, 8, _lib.DT_F32, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # f32 rows, split into bf16 parts
+  assert d(127, 14336, 4096, 4096, 8, _lib.DT_F32, 0) == _lib.KERNEL_SKINNY_MFMA         # fewer than 128: 16 per pass
+  assert d(128, 14336, 4096, 4096, 8, _lib.DT_F32, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM
+  assert d(2048, 14336, 4096 + 64, 4096 + 64, 8, _lib.DT_F32, 0) == _lib.KERNEL_GENERIC
+  assert lib.xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(2048, 14336, 4096) == 2048 * 4096 * 6
+  assert lib.xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(2048, 14336, 4100) == 0
   assert d(2048, 4096, 4096, 128, 8, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # blockwise: its own tiled GEMM
   assert d(2048, 14336, 4096, 4096, 4, _lib.DT_BF16, 0) == _lib.KERNEL_WEIGHT_ONLY_GEMM  # int4 too
   assert d(64, 4096, 4096, 128, 4, _lib.DT_BF16, 0) == _lib.KERNEL_SKINNY_MFMA         # up to 64 rows stream (two passes)

@@ -17,7 +17,7 @@ OVERFLOW_SATURATE, OVERFLOW_WRAP = 0, 1
 W_NK, W_SCN = 0, 1
 QDT_I8, QDT_U8, QDT_I16, QDT_I32 = 0, 1, 2, 3
 KERNEL_GENERIC, KERNEL_SKINNY_MFMA, KERNEL_W8A8_MFMA, KERNEL_W8A8_GENERIC, KERNEL_WEIGHT_ONLY_GEMM = 0, 1, 2, 3, 4
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _DT = {torch.float32: DT_F32, torch.bfloat16: DT_BF16, torch.float16: DT_F16}
 
@@ -36,6 +36,8 @@ SIGNATURES = {
     "xla_amd_qmm_weight_only_skinny": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),
     "xla_amd_qmm_weight_only_gemm_workspace_bytes": (ctypes.c_size_t, [_c_i64] * 4 + [_c_int]),
     "xla_amd_qmm_weight_only_gemm": (_c_int, [_c_vp] * 6 + [ctypes.c_size_t] + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),
+    "xla_amd_qmm_weight_only_gemm_f32_workspace_bytes": (ctypes.c_size_t, [_c_i64] * 3),
+    "xla_amd_qmm_weight_only_gemm_f32": (_c_int, [_c_vp] * 6 + [ctypes.c_size_t] + [_c_i64] * 3 + [_c_int] * 2 + [_c_vp]),
     "xla_amd_qmm_weight_only_generic": (_c_int, [_c_vp] * 5 + [_c_i64] * 4 + [_c_int] * 7 + [_c_vp]),
     "xla_amd_qmm_quantize_per_token": (_c_int, [_c_vp] * 4 + [_c_i64] * 2 + [_c_int] * 3 + [_c_vp]),
     "xla_amd_qmm_w8a8_gemm": (_c_int, [_c_vp] * 8 + [_c_i64] * 3 + [_c_int] * 9 + [_c_vp]),

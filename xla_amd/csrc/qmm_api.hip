@@ -132,6 +132,10 @@ extern "C" int xla_amd_qmm_dispatch(int64_t M, int64_t N, int64_t K, int64_t C, 
   // many rows of 2-byte x against per-channel int8 weights: the tiled GEMM reads the weight once
   // per 128 rows, the streaming kernel once per 32
   if (C == K && bits == 8 && K % 128 == 0 && x_dt != XLA_AMD_DT_F32 && M > 32) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
+  // many rows of f32 x: the same GEMM over x split into three bf16 parts (xla_amd_qmm_weight_only_gemm_f32), three
+  // times the arithmetic, where the streaming kernel makes a pass over the weight for every 16 rows (from 128 rows
+  // on: 4096 x 4096 takes 103 us either way there, 14336 x 4096 118 against 250 us)
+  if (C == K && bits == 8 && K % 128 == 0 && 3 * K <= (1 << 23) && x_dt == XLA_AMD_DT_F32 && M >= 128) return XLA_AMD_KERNEL_WEIGHT_ONLY_GEMM;
   // few rows against few channels and a long K: the streaming kernel over K slices, behind the GEMM's entry point
   if ((bits == 8 || bits == 4) && x_dt != XLA_AMD_DT_F32 && K % C == 0) {
     int per;

@@ -56,6 +56,8 @@ struct WoGemmArgs {
   int k_per_split;     // columns per K slice (a multiple of 128)
   int split;
   int scale_dt, zp_dt, dot_dt, out_dt, store_dt;
+  int Kw;    // columns of the weight: K, or K / 3 when x is an f32 matrix split into three bf16 parts side by side
+  int x_dt;  // the caller's x dtype (the row sums of x are rounded to it): the kernel's, or f32 for split f32 rows
 };
 
 // one launcher per unit: row tile of 16 * MT rows, ng = 2 or 4 channel groups per computing wave
@@ -93,10 +95,10 @@ template <int MT, int NG> struct WoCfg {
 // The dtypes of the epilogue: those of the call, or (UNI) all equal to x's dtype and known at
 // compile time, which is the common case and removes every branch on a dtype.
 template <int XT, bool UNI> struct WoDts {
-  int scale_dt, zp_dt, dot_dt, out_dt, store_dt;
+  int scale_dt, zp_dt, dot_dt, out_dt, store_dt, x_dt;
   __device__ __forceinline__ explicit WoDts(const WoGemmArgs& a)
       : scale_dt(UNI ? XT : a.scale_dt), zp_dt(UNI ? XT : a.zp_dt), dot_dt(UNI ? XT : a.dot_dt),
-        out_dt(UNI ? XT : a.out_dt), store_dt(UNI ? XT : a.store_dt) {}
+        out_dt(UNI ? XT : a.out_dt), store_dt(UNI ? XT : a.store_dt), x_dt(UNI ? XT : a.x_dt) {}
 };
 
 // Scale (or zero point) of four consecutive channels as raw bits; channels past N repeat the last one.
@@ -270,7 +272,8 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   // channels, whatever the width G of the channel groups of the tiled weight: channel n lies in group n / G at
   // row n % G, so the 16 rows of a set come out of one or two groups and every lane keeps its own offset
   // (channels past N read the last one again; their results are dropped).
-  const int n_blk = K / 128;  // blocks per channel group in the tiled weight
+  const int n_blk = a.Kw / 128;  // blocks per channel group in the tiled weight
+  const int w_halves = 2 * n_blk;  // the item's halves wrap round the weight's (x in three parts: three trips)
   const int blk_bytes = G * 128, half_bytes = G * 64;
   constexpr int H = wo_ring_halves<MT, NG, HASZP, UNI>(), R = Cfg::R;
   static_assert(H % 2 == 1, "a step uses two halves: an odd ring visits every phase in H steps");
@@ -291,7 +294,9 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   // around the loads: the counts of loads in flight stay known at compile time on every path)
   auto request = [&](int q, int last, auto slotc) __attribute__((always_inline)) {
     constexpr int slot = slotc;
-    const int qq = min(q, last);
+    int qq = min(q, last);
+    if (qq >= w_halves) qq -= w_halves;
+    if (qq >= w_halves) qq -= w_halves;
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
       const uint8_t* half = wp + (size_t)qq * half_bytes;  // uniform: scalar base + lane offset
@@ -429,12 +434,12 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
                   wo_finish_store_bf16(a.out, m, n, N, sraw[gi], acc[gi][mt]);
                 } else {
                   float o[4];
-                  wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, XT, o);
+                  wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, dts.x_dt, o);
                   wo_store4<kVec>(a.out, m, n, N, o, dts.store_dt);
                 }
               } else {
                 float o[4];
-                wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, XT, o);
+                wo_finish4(dts, sraw[gi], zraw[gi], HASZP, acc[gi][mt], HASZP ? xs[mt][0] : 0.f, dts.x_dt, o);
                 wo_store_some(a.out, m, n, N, cnt, o, dts.store_dt);
               }
             }
@@ -641,6 +646,77 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
 
 }  // namespace
 
+namespace {
+
+// x f32 [M, K] -> [M, 3 K] bf16: hi | mid | lo side by side, hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid)
+// (round to nearest even; the differences are exact in f32): hi + mid + lo = x to the last bit of f32 for finite x,
+// and every product of a part with an int8 weight is exact in the f32 accumulator of the MFMA.  An infinity or a
+// NaN stays in hi alone.
+__global__ void __launch_bounds__(256) qmm_split3_kernel(const float* x, uint16_t* out, int64_t quads, int K) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= quads) return;
+  const int kq = K / 4;
+  const int64_t m = i / kq;
+  const int c = (int)(i - m * kq) * 4;
+  const f32x4 v = *(const f32x4*)(x + m * K + c);
+  uint16_t part[3][4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const uint16_t hi = qmm_f32_to_bf16(v[e]);
+    const float fh = qmm_bf16_to_f32(hi);
+    const bool finite = (__float_as_uint(fh) & 0x7f800000u) != 0x7f800000u;
+    const float r1 = finite ? v[e] - fh : 0.f;
+    const uint16_t mid = qmm_f32_to_bf16(r1);
+    const float r2 = r1 - qmm_bf16_to_f32(mid);
+    part[0][e] = hi; part[1][e] = mid; part[2][e] = qmm_f32_to_bf16(r2);
+  }
+  uint16_t* o = out + m * (3 * (int64_t)K) + c;
+#pragma unroll
+  for (int t = 0; t < 3; ++t)
+    *(i32x2*)(o + (int64_t)t * K) = i32x2{(int)(part[t][0] | ((uint32_t)part[t][1] << 16)), (int)(part[t][2] | ((uint32_t)part[t][3] << 16))};
+}
+
+}  // namespace
+
+extern "C" size_t xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  return (size_t)M * (size_t)K * 3 * sizeof(uint16_t);
+}
+
+extern "C" int xla_amd_qmm_weight_only_gemm_f32(const float* x, const void* w_tiled, const void* scale, const void* zp,
+                                                float* out, void* workspace, size_t workspace_bytes, int64_t M, int64_t N,
+                                                int64_t K, int scale_dt, int zp_dt, void* stream) {
+  if (!x || !w_tiled || !scale || !out) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm_f32: null pointer");
+  if (M < 0 || N <= 0 || K <= 0) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm_f32: bad sizes");
+  if (!qmm_valid_dt(scale_dt) || (zp && !qmm_valid_dt(zp_dt))) return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm_f32: bad dtype enum");
+  if (K % 128 != 0) return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm_f32: K=%lld must be a multiple of 128", (long long)K);
+  if (N > (1 << 30) || 3 * K > (1 << 23) || M > (1 << 24))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm_f32: dimension too large");
+  if ((((uintptr_t)x | (uintptr_t)w_tiled | (uintptr_t)out | (uintptr_t)workspace) & 15))
+    return qmm_fail(XLA_AMD_QMM_EUNSUPPORTED, "weight_only_gemm_f32: x, w, out and workspace must be 16-byte aligned");
+  if (M == 0) return XLA_AMD_QMM_OK;
+  const size_t need = xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(M, N, K);
+  if (!workspace || workspace_bytes < need)
+    return qmm_fail(XLA_AMD_QMM_EINVAL, "weight_only_gemm_f32: workspace of %zu bytes, need %zu", workspace ? workspace_bytes : (size_t)0, need);
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t quads = M * (K / 4);
+  hipLaunchKernelGGL(qmm_split3_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, x, (uint16_t*)workspace, quads, (int)K);
+  int rc = QMM_CHECK_LAUNCH("weight_only_gemm_f32 split launch");
+  if (rc != XLA_AMD_QMM_OK) return rc;
+  // the bf16 GEMM over 3 K columns of x against the weight's K columns three times over, f32 from the dot product on
+  Plan p = make_plan(M, N, 3 * K, zp != nullptr);
+  WoGemmArgs a;
+  a.x = workspace; a.w = (const uint8_t*)w_tiled; a.scale = scale; a.zp = zp; a.out = out;
+  a.part = nullptr; a.part_xs = nullptr;
+  a.M = (int)M; a.N = (int)N; a.K = (int)(3 * K);
+  a.Kw = (int)K; a.x_dt = XLA_AMD_DT_F32;
+  a.G = xla_amd_qmm_tile_group(N, K, K, 8);
+  a.k_per_split = (int)(3 * K); a.split = 1;  // (no K split: a slice would have to wrap round the weight)
+  a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : XLA_AMD_DT_F32;
+  a.dot_dt = XLA_AMD_DT_F32; a.out_dt = XLA_AMD_DT_F32; a.store_dt = XLA_AMD_DT_F32;
+  return p.mt == 4 ? qmm_wo_launch_bf16_mt4(a, p.ng, s) : qmm_wo_launch_bf16_mt8(a, p.ng, s);
+}
+
 extern "C" size_t xla_amd_qmm_weight_only_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t C, int bits) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
   if (C <= 0) C = K;
@@ -752,6 +828,7 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
   a.x = x; a.w = (const uint8_t*)w_tiled; a.scale = scale; a.zp = zp; a.out = out;
   a.part = nullptr; a.part_xs = nullptr;
   a.M = (int)M; a.N = (int)N; a.K = (int)K;
+  a.Kw = (int)K; a.x_dt = x_dt;
   a.G = xla_amd_qmm_tile_group(N, K, K, 8);
   a.k_per_split = p.k_per_split; a.split = p.split;
   a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.dot_dt = dot_dt; a.out_dt = out_dt; a.store_dt = store_dt;

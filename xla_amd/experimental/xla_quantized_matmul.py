@@ -228,6 +228,21 @@ def _weight_only_launch(x2, w, w_tiled, n, k, c, layout, bits, scaler, zero_poin
             dot_dtype == x2.dtype and out_dtype == x2.dtype and store_dtype == x2.dtype)
     if not same:
       kern = _lib.KERNEL_SKINNY_MFMA
+  if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM and x2.dtype == torch.float32:
+    if store_dtype != torch.float32 or dot_dtype != torch.float32:
+      kern = _lib.KERNEL_SKINNY_MFMA  # (f32 rows with a narrower stored result: no caller; the streaming kernel does it)
+    else:
+      # f32 rows: split into three bf16 parts in a workspace, then the bf16 GEMM with f32 accumulation throughout
+      wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
+      counters["wo_gemm"] += 1
+      nbytes = lib.xla_amd_qmm_weight_only_gemm_f32_workspace_bytes(m, n, k)
+      workspace = torch.empty(nbytes, dtype=torch.uint8, device=x2.device)
+      x2 = x2.contiguous()
+      _lib.check(
+          lib.xla_amd_qmm_weight_only_gemm_f32(x2.data_ptr(), wk.data_ptr(), scaler.data_ptr(), _lib.ptr(zero_point),
+                                               out.data_ptr(), workspace.data_ptr(), nbytes, m, n, k,
+                                               _lib.dt(scaler.dtype), zp_dt, stream), "weight_only_gemm_f32")
+      return out
   if kern == _lib.KERNEL_WEIGHT_ONLY_GEMM:
     wk = w_tiled if w_tiled is not None else _tiled_weight(w, bits, layout)
     counters["wo_gemm"] += 1
