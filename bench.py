@@ -492,7 +492,15 @@ def main():
                      "kernel": "qmm_wo_gemm_kernel<bf16, 128 x 256 tile> (persistent, 4 computing + 4 copying waves)"},
         "vs_w8a8_end_to_end": round(ev_wo / ev_e2e, 2),
     }
-    del x4, x4b, xq, xsc
+    # the same shape with f32 activations: split into three bf16 parts, the same GEMM at three times the arithmetic
+    x4f = torch.randn(m4, K_IN, generator=cases.gen(2)).to(dev)
+    s2f = s2.float()
+    _, ev_f32, _ = time_calls([lambda: op(x4f, w0, s2f)], 10, 3, use_graph)
+    extra["weight_only_prefill_M2048_f32_rows"] = {
+        "us": round(ev_f32 * 1e3, 1),
+        "note": "x f32 [2048,4096]: xla_amd_qmm_weight_only_gemm_f32 (split kernel + bf16 GEMM over 3 K columns, f32 results; "
+                "workspace allocation included); the streaming kernel's 128 passes take 3.8 ms"}
+    del x4, x4b, x4f, xq, xsc
 
     # Llama-3-8B decoder layer, 7 linears (config 5)
     shapes = {"q": (4096, 4096), "k": (1024, 4096), "v": (1024, 4096), "o": (4096, 4096),
