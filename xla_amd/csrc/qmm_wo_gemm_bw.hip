@@ -150,7 +150,8 @@ qmm_wo_bw_gemm_kernel(WoBwArgs a) {
       constexpr int gi = gc;
       qmm_static_for<WL>([&](auto hc) {
         constexpr int h = hc;
-        wnext[gi][h] = __builtin_nontemporal_load((const i32x4*)(wp[gi] + (size_t)blk * BLK + h * 1024));
+        // (an ordinary load, not a streaming one: the other row tiles read the same block out of L2)
+        wnext[gi][h] = *(const i32x4*)(wp[gi] + (size_t)blk * BLK + h * 1024);
       });
     });
   };
