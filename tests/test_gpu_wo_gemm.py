@@ -184,6 +184,30 @@ def test_wo_gemm_several_rounds_of_tiles(ops, xdt):
     check(out, exp, f"several rounds {m,n,k}")
 
 
+@pytest.mark.parametrize("xdt", [torch.bfloat16, torch.float16])
+def test_wo_gemm_results_written_out_by_the_copying_waves(ops, xdt):
+  """From 12 steps of K up, with one 2-byte dtype throughout and N a multiple of 8, the 128 x 256 tile leaves its
+  results in LDS and the copying waves scale them and write them out during the next item: exactly 12 and 13 steps,
+  one item per workgroup and several, row and column tails."""
+  for (m, n, k) in [(1024, 8192, 1536), (1100, 7496, 1664), (2048, 14336, 1536)]:
+    x, w, s, _ = cases.per_channel_int8(m, n, k, xdt, xdt, seed=m + k)
+    exp = oracle.quantized_matmul(x, w, s)
+    out = wo_gemm(ops, x.cuda(), w.cuda(), s.cuda(), None)
+    check(out, exp, f"results through LDS {m,n,k}")
+    if m == 1100:  # the same with a scale vector that does not start on 16 bytes: the computing waves store
+      out2 = torch.empty(m, n, dtype=xdt, device="cuda")
+      s2 = torch.empty(n + 4, dtype=xdt, device="cuda")[4:].copy_(s)
+      assert s2.data_ptr() % 16 != 0
+      lib = _lib.load()
+      assert lib.xla_amd_qmm_weight_only_gemm_workspace_bytes(m, n, k, k, 8) == 0
+      wt = ops._tiled_weight(w.cuda(), 8, _lib.W_NK)
+      rc = lib.xla_amd_qmm_weight_only_gemm(x.cuda().data_ptr(), wt.data_ptr(), s2.data_ptr(), None, out2.data_ptr(), None, 0,
+                                            m, n, k, k, 8, _lib.dt(xdt), _lib.dt(xdt), _lib.dt(xdt), _lib.dt(xdt), _lib.dt(xdt),
+                                            _lib.dt(xdt), torch.cuda.current_stream().cuda_stream)
+      _lib.check(rc, "weight_only_gemm")
+      assert torch.equal(out2, out)
+
+
 @pytest.mark.parametrize("sdt", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("zp", [False, True])
 def test_f32_rows_through_the_tiled_gemm(ops, sdt, zp):

@@ -58,6 +58,7 @@ struct WoGemmArgs {
   int scale_dt, zp_dt, dot_dt, out_dt, store_dt;
   int Kw;    // columns of the weight: K, or K / 3 when x is an f32 matrix split into three bf16 parts side by side
   int x_dt;  // the caller's x dtype (the row sums of x are rounded to it): the kernel's, or f32 for split f32 rows
+  int stage_out;  // 128 x 256 tile: results leave through LDS, written out by the copying waves during the next item
 };
 
 // one launcher per unit: row tile of 16 * MT rows, ng = 2 or 4 channel groups per computing wave
@@ -85,11 +86,16 @@ template <int MT, int NG, bool HASZP, bool UNI> constexpr int wo_ring_halves() {
 template <int MT, int NG> struct WoCfg {
   static constexpr int BM = 16 * MT;
   static constexpr int X_TILE = BM * 256;  // bytes of the x columns of one step (128 columns, 2-byte x)
+  // The 128 x 256 tile keeps room for its 2-byte results in LDS (64 KB): the computing waves leave them there and
+  // go on with the next item, and the copying waves write them out a little per step.  Stored by the computing
+  // waves themselves, the 16.8 MB that all workgroups finish at the same moment cost 6 - 8 us per item, during which
+  // nothing is computed (a build without the stores: 249 -> 223 us).
+  static constexpr int kStage = (MT == 8 && NG == 4) ? BM * 64 * NG * 2 : 0;
   // x tiles (one step each) in LDS: a ring that the copying waves fill R - 1 tiles ahead of the computing waves
-  static constexpr int kFit = kLds / X_TILE;
+  static constexpr int kFit = (kLds - kStage) / X_TILE;
   static constexpr int R = kFit < 8 ? kFit : 8;
   static_assert(R >= 3, "the x ring needs room to run ahead");
-  static constexpr int lds_bytes(int steps) { return (steps < R ? steps : R) * X_TILE; }
+  static constexpr int lds_bytes(int steps) { return kStage + (steps < R ? steps : R) * X_TILE; }
 };
 
 // The dtypes of the epilogue: those of the call, or (UNI) all equal to x's dtype and known at
@@ -174,14 +180,17 @@ __device__ __forceinline__ void wo_store_some(void* out, int m, int n, int N, in
 
 // The same epilogue and store when every dtype is bf16 and there is no zero point: two
 // values per conversion, and the rounded product is already the stored bit pattern.
-__device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, int N, const uint32_t sraw[4], f32x4 dot) {
-  uint32_t res[2];
+__device__ __forceinline__ void wo_finish_pack_bf16(const uint32_t sraw[4], f32x4 dot, uint32_t res[2]) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const uint32_t p = qmm_f32x2_to_bf16x2(dot[2 * h], dot[2 * h + 1]);
     const float p0 = __uint_as_float(p << 16), p1 = __uint_as_float(p & 0xffff0000u);
     res[h] = qmm_f32x2_to_bf16x2(__uint_as_float(sraw[2 * h] << 16) * p0, __uint_as_float(sraw[2 * h + 1] << 16) * p1);
   }
+}
+__device__ __forceinline__ void wo_finish_store_bf16(void* out, int m, int n, int N, const uint32_t sraw[4], f32x4 dot) {
+  uint32_t res[2];
+  wo_finish_pack_bf16(sraw, dot, res);
   *(i32x2*)((uint16_t*)out + (size_t)m * N + n) = i32x2{(int)res[0], (int)res[1]};
 }
 
@@ -201,6 +210,8 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   constexpr int BM = Cfg::BM, X_TILE = Cfg::X_TILE;
   constexpr int BN = 64 * NG;  // channels per workgroup: NG MFMA row sets of 16 per computing wave
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* const ring = smem + Cfg::kStage;  // the x tiles; before them the results on their way out
+  const bool stage_out = Cfg::kStage > 0 && a.stage_out != 0;
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
   const int lane = threadIdx.x & 63;
@@ -236,33 +247,129 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     for (int i = blockIdx.x; i < n_items; i += gridDim.x) total += item_of(i).steps;
     int q_it = blockIdx.x, q_s = 0, issued = 0;  // the next tile to request: step q_s of item q_it
     WoItem q = item_of(q_it);
-    auto issue = [&]() __attribute__((always_inline)) {
-      if (issued >= total) return;
-      char* const dst = smem + (issued % R) * X_TILE;
-      const char* const xb = (const char*)a.x + ((size_t)q.m0 * K + q.k_begin) * 2 + (size_t)q_s * 256;
+    // this lane's part of each of its L loads of a tile, from the tile's first byte (less than 2^32: 128 rows of at
+    // most 2^24 bytes): lane l copies row l / 16 of four, 16-byte chunk l % 16, swizzled on the source side; rows
+    // past the end repeat the last one.  Kept across the steps of an item: the base of a tile is then scalar.
+    uint32_t x_off[L];
+    auto set_offsets = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < L; ++i) {
-        // (lane l: row l / 16 of the four, 16-byte chunk l % 16, swizzled on the source side;
-        // rows past the end repeat the last one)
-        const int r4 = (cw + i * kCopyWaves) * 4;
-        const int row = min(r4 + (lane >> 4), q.rows - 1);
-        const int chunk = (lane & 15) ^ (row & 15);
-        __builtin_amdgcn_global_load_lds((const void*)(xb + (size_t)row * ((size_t)K * 2) + chunk * 16),
-                                         (lds_ptr_t)(dst + r4 * 256), 16, 0, 0);
+        const int row = min((cw + i * kCopyWaves) * 4 + (lane >> 4), q.rows - 1);
+        x_off[i] = (uint32_t)row * ((uint32_t)K * 2u) + (uint32_t)(((lane & 15) ^ (row & 15)) * 16);
       }
+    };
+    set_offsets();
+    auto issue = [&]() __attribute__((always_inline)) {
+      if (issued >= total) return;
+      char* const dst = ring + (issued % R) * X_TILE;
+      const char* const xb = (const char*)a.x + ((size_t)q.m0 * K + q.k_begin) * 2 + (size_t)q_s * 256;
+#pragma unroll
+      for (int i = 0; i < L; ++i)
+        __builtin_amdgcn_global_load_lds((const void*)(xb + (size_t)x_off[i]), (lds_ptr_t)(dst + (cw + i * kCopyWaves) * 1024), 16, 0, 0);
       ++issued;
       if (++q_s == q.steps) {
         q_s = 0;
         q_it += gridDim.x;
-        if (q_it < n_items) q = item_of(q_it);
+        if (q_it < n_items) {
+          const int rows_before = q.rows;
+          q = item_of(q_it);
+          if (q.rows != rows_before) set_offsets();
+        }
       }
     };
+    // Results that the computing waves left in LDS (stage_out): the dot products rounded to the dot dtype,
+    // [128 rows][256 channels] of 2 bytes, the 16-byte chunks of a row swizzled by the row.  The copying waves
+    // multiply them by the channels' scales and write them out: an instruction two rows (512 bytes each: whole
+    // lines); a wave has 16 of them per item and does two per step from the next item's first step on.  A lane
+    // always handles the same eight channels of the tile and keeps their scales in registers.  These reach it
+    // through LDS as well (a load into registers here would make the compiler wait for every x tile in flight):
+    // with the results written out, four steps before the item's end, the first copying wave requests the item's
+    // 256 scales into the first row of the results' area; two steps later, a barrier after they have arrived, every
+    // copying wave reads its lanes' scales, and another barrier later the computing waves may overwrite them.
+    // The host asks for this path from 12 steps per item up.
+    constexpr int kDrainPerWave = BM / 2 / kCopyWaves;
+    static_assert(Cfg::kStage == 0 || D == 2, "the waits below count what is issued within one step");
+    int c_it = blockIdx.x, c_s = 0, drain_left = 0;  // the step the computing waves begin after the next barrier
+    WoItem c_item = item_of(c_it), d_item = c_item;  // d_item: the item whose results are in LDS
+    float sc[8] = {0, 0, 0, 0, 0, 0, 0, 0};          // scales of the channels n0 + 8 (lane % 32) .. + 7 of d_item
+    // (the LDS reads are written as assembly: the compiler would put a wait for every load of x in flight before
+    // an LDS read that follows them in the same wave, since those loads write LDS)
+    auto lds_read16 = [&](const char* p) __attribute__((always_inline)) {
+      i32x4 v;
+      asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(v) : "v"((uint32_t)(uintptr_t)(lds_ptr_t)p) : "memory");
+      return v;
+    };
+    // Writes out up to two pairs of rows and returns the number of store instructions issued (a pair of rows
+    // past M issues none).
+    auto drain = [&]() __attribute__((always_inline)) {
+      int stores = 0;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (drain_left > 0) {
+          const int pair = cw * kDrainPerWave + (kDrainPerWave - drain_left);  // uniform over the wave
+          --drain_left;
+          if (d_item.m0 + 2 * pair < M) {
+            const int row = 2 * pair + (lane >> 5), c = lane & 31;
+            const i32x4 v = lds_read16(smem + row * 512 + ((c ^ (row & 31)) * 16));
+            i32x4 o;
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+              const uint32_t d = (uint32_t)v[h];
+              const float r0 = sc[2 * h] * qmm_from_raw(d & 0xffffu, XT), r1 = sc[2 * h + 1] * qmm_from_raw(d >> 16, XT);
+              o[h] = (int)(XT == XLA_AMD_DT_BF16 ? qmm_f32x2_to_bf16x2(r0, r1) : qmm_f32x2_to_f16x2(r0, r1));
+            }
+            const int m = d_item.m0 + row, n = d_item.n0 + 8 * c;
+            if (m < M && n < N) *(i32x4*)((uint16_t*)a.out + (size_t)m * N + n) = o;
+            ++stores;
+          }
+        }
+      }
+      return stores;
+    };
     for (int d = 0; d < D; ++d) issue();
+    int ops_before = 0;  // memory instructions issued between the loads of tile n and those of tile n + 1
     for (int n = 0; n < total; ++n) {
-      if (issued - n == D) qmm_wait_vmcnt<(D - 1) * L>();  // the tiles n + 1 .. n + D - 1 may be in flight
-      else qmm_wait_vmcnt<0>();                             // (the first and the last tiles of the workgroup)
+      // the tiles n + 1 .. n + D - 1 may be in flight, and what was issued between them (the memory instructions
+      // of a wave complete in the order of their issue)
+      if (issued - n == D) {
+        if (ops_before == 0) qmm_wait_vmcnt<(D - 1) * L>();
+        else if (ops_before == 1) qmm_wait_vmcnt<(D - 1) * L + 1>();
+        else qmm_wait_vmcnt<(D - 1) * L + 2>();
+      } else {
+        qmm_wait_vmcnt<0>();  // (the first and the last tiles of the workgroup)
+      }
       qmm_bare_barrier();  // tile n is there; the computing waves have read tile n - 1
-      issue();             // tile n + D into the slot of tile n - 1
+      ops_before = 0;
+      if (stage_out) {
+        if (c_s < c_item.steps - 4) {
+          ops_before = drain();
+        } else if (c_s == c_item.steps - 4) {
+          if (cw == 0) {  // (lanes 32 .. 63 fetch the same 512 bytes again, into the second row)
+            const int n8 = min(c_item.n0 + 8 * (lane & 31), N - 8);
+            __builtin_amdgcn_global_load_lds((const void*)((const uint16_t*)a.scale + n8), (lds_ptr_t)smem, 16, 0, 0);
+            ops_before = 1;
+          }
+        } else if (c_s == c_item.steps - 2) {
+          const i32x4 v = lds_read16(smem + (lane & 31) * 16);
+#pragma unroll
+          for (int h = 0; h < 4; ++h) {
+            sc[2 * h] = qmm_from_raw((uint32_t)v[h] & 0xffffu, XT);
+            sc[2 * h + 1] = qmm_from_raw((uint32_t)v[h] >> 16, XT);
+          }
+        }
+        if (++c_s == c_item.steps) {  // after this step the computing waves leave this item's results in LDS
+          d_item = c_item;
+          drain_left = kDrainPerWave;
+          c_s = 0;
+          c_it += gridDim.x;
+          if (c_it < n_items) c_item = item_of(c_it);
+        }
+      }
+      issue();  // tile n + D into the slot of tile n - 1
+    }
+    if (stage_out) {
+      qmm_bare_barrier();  // the last item's results are in LDS
+      while (drain_left > 0) drain();
     }
     return;
   }
@@ -321,7 +428,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   // the conversions, and with one computing wave per SIMD nothing else fills the gap.
   auto compute = [&](int xslot, int s, int S, auto phc) __attribute__((always_inline)) {
     constexpr int PH = phc;
-    const char* xrow = smem + xslot * X_TILE + r * 256;  // this lane's row of each 16-row tile
+    const char* xrow = ring + xslot * X_TILE + r * 256;  // this lane's row of each 16-row tile
     const int last = 2 * S - 1;
     auto xfrag = [&](int j, int mt) __attribute__((always_inline)) {
       return *(const i32x4*)(xrow + mt * (16 * 256) + (((4 * g + j) ^ r) * 16));
@@ -406,7 +513,22 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       n = n_first + gi * 16;
       cnt = min(N - n, 4);
     };
-    if (a.split == 1) {
+    if (stage_out) {
+      // the dot products, rounded, into LDS: row 16 mt + r, 16-byte chunk 8 wave + 2 gi + g / 2 (swizzled by the
+      // row), half g % 2; the copying waves scale them and write them out
+      qmm_static_for<MT>([&](auto mc) {
+        constexpr int mt = mc;
+        const int row = 16 * mt + r;
+        qmm_static_for<NG>([&](auto gc) {
+          constexpr int gi = gc;
+          const f32x4 d = acc[gi][mt];
+          const uint32_t lo = XT == XLA_AMD_DT_BF16 ? qmm_f32x2_to_bf16x2(d[0], d[1]) : qmm_f32x2_to_f16x2(d[0], d[1]);
+          const uint32_t hi = XT == XLA_AMD_DT_BF16 ? qmm_f32x2_to_bf16x2(d[2], d[3]) : qmm_f32x2_to_f16x2(d[2], d[3]);
+          const int chunk = (wave * 8 + gi * 2 + (g >> 1)) ^ (row & 31);
+          *(i32x2*)(smem + row * 512 + chunk * 16 + (g & 1) * 8) = i32x2{(int)lo, (int)hi};
+        });
+      });
+    } else if (a.split == 1) {
       const WoDts<XT, UNI> dts(a);
       // scales (and zero points) of this lane's channels first, all at once: loads inside the
       // loop over row tiles would be waited for one after the other
@@ -447,8 +569,11 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
           });
         });
       };
-      if ((N & 3) == 0) emit(qmm_const<1>{});
-      else emit(qmm_const<0>{});
+      if ((N & 3) == 0) {
+        emit(qmm_const<1>{});
+      } else {
+        emit(qmm_const<0>{});
+      }
     } else {
       const bool vec = (N & 3) == 0;
       qmm_static_for<NG>([&](auto gc) {
@@ -478,6 +603,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
     }
     if (!more) break;
   }
+  if (stage_out) qmm_bare_barrier();  // the copying waves may write out the last item's results
 }
 
 // Compute units of the current device (asked once per device).
@@ -710,7 +836,7 @@ extern "C" int xla_amd_qmm_weight_only_gemm_f32(const float* x, const void* w_ti
   a.x = workspace; a.w = (const uint8_t*)w_tiled; a.scale = scale; a.zp = zp; a.out = out;
   a.part = nullptr; a.part_xs = nullptr;
   a.M = (int)M; a.N = (int)N; a.K = (int)(3 * K);
-  a.Kw = (int)K; a.x_dt = XLA_AMD_DT_F32;
+  a.Kw = (int)K; a.x_dt = XLA_AMD_DT_F32; a.stage_out = 0;
   a.G = xla_amd_qmm_tile_group(N, K, K, 8);
   a.k_per_split = (int)(3 * K); a.split = 1;  // (no K split: a slice would have to wrap round the weight)
   a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : XLA_AMD_DT_F32;
@@ -832,6 +958,11 @@ extern "C" int xla_amd_qmm_weight_only_gemm(const void* x, const void* w_tiled, 
   a.Kw = (int)K; a.x_dt = x_dt;
   a.G = xla_amd_qmm_tile_group(N, K, K, 8);
   a.k_per_split = p.k_per_split; a.split = p.split;
+  // (results through LDS: the 128 x 256 tile with one 2-byte dtype throughout, whole 16-byte chunks per row of the
+  // output and of the scales, and enough steps per item for the copying waves to write an item's results out during
+  // the next one and to fetch the scales after that)
+  a.stage_out = p.mt == 8 && p.ng == 4 && p.split == 1 && !zp && scale_dt == x_dt && dot_dt == x_dt && out_dt == x_dt &&
+                store_dt == x_dt && N % 8 == 0 && K / 128 >= 12 && ((((uintptr_t)out) | ((uintptr_t)scale)) & 15) == 0;
   a.scale_dt = scale_dt; a.zp_dt = zp ? zp_dt : x_dt; a.dot_dt = dot_dt; a.out_dt = out_dt; a.store_dt = store_dt;
   if (p.split > 1) {
     const size_t need = ((size_t)p.split * (size_t)M * (size_t)N + (size_t)p.split * (size_t)M) * sizeof(float);
