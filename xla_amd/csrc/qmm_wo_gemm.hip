@@ -416,53 +416,58 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   };
 
   f32x4 acc[NG][MT], xs[MT];
+  // The converted weight fragments of one j (columns 32 g + 8 j .. + 7 of the step, one fragment per row set gi):
+  // those in use and those of the next j, which are converted meanwhile; the fragments of a step's first j are
+  // converted during the step before (or, for an item's first step, by prime()).
+  i32x4 af[2][NG];
+  auto prime = [&]() __attribute__((always_inline)) {
+    qmm_static_for<NG>([&](auto gc) {
+      const i32x4 src = wreg[0][(int)gc];
+      af[0][(int)gc] = cvt_w8<XT>((uint32_t)src[0], (uint32_t)src[1]);
+    });
+  };
   // One step (128 columns): step s of an item of S steps, x out of LDS slot `xslot`, weights out of the ring
   // slots PH (columns 0 .. 63) and PH + 1 (columns 64 .. 127); each slot is requested again (half + H of the
-  // item) as soon as it has been used.
-  // The step is software-pipelined by hand over its 4 * NG weight fragments (fragment f = j * NG + gi: columns
-  // 32 g + 8 j .. of channel group gi).  Between the MT MFMAs of fragment f sit the conversions of fragment f + 1
-  // (a quarter of them, three instructions, after every MT / 4 th MFMA: about what fits in the issue slots that an
-  // MFMA leaves free), and in the last group of a j every MFMA is followed by the LDS read that replaces its x
-  // fragment with that of j + 1.  A scheduling fence after each such unit keeps the order: left to itself the
-  // compiler emits the conversions and the MFMAs of a fragment as two separate runs, the matrix pipe idles during
-  // the conversions, and with one computing wave per SIMD nothing else fills the gap.
+  // item) as soon as its last fragment has been converted.
+  // The order is j, row tile mt, row set gi: an x fragment (one LDS read) serves NG MFMAs in a row and is read two
+  // row tiles ahead into one of three registers in turn, so the LDS reads of the four computing waves, which run
+  // in step, come one per NG MFMAs instead of MT at once (that burst, 32 KB per compute unit, took longer than
+  // the MFMAs it fed: a quarter of the step went to waiting for LDS).  Between the MFMAs sit the conversions of
+  // the next j's fragments, a quarter of a fragment (three instructions) after every MT / 4 th MFMA.  A
+  // scheduling fence after each MFMA keeps that order: left to itself the compiler emits the conversions and
+  // the MFMAs as separate runs, and with one computing wave per SIMD nothing else fills the gaps.
   auto compute = [&](int xslot, int s, int S, auto phc) __attribute__((always_inline)) {
     constexpr int PH = phc;
     const char* xrow = ring + xslot * X_TILE + r * 256;  // this lane's row of each 16-row tile
     const int last = 2 * S - 1;
-    auto xfrag = [&](int j, int mt) __attribute__((always_inline)) {
-      return *(const i32x4*)(xrow + mt * (16 * 256) + (((4 * g + j) ^ r) * 16));
+    auto xfrag = [&](int idx) __attribute__((always_inline)) {  // idx = j * MT + mt
+      return *(const i32x4*)(xrow + (idx % MT) * (16 * 256) + (((4 * g + idx / MT) ^ r) * 16));
     };
-    i32x4 xq[MT];
-    qmm_static_for<MT>([&](auto mc) { xq[(int)mc] = xfrag(0, mc); });
-    i32x4 af;
-    {
-      const i32x4 src = wreg[PH][0];
-      af = cvt_w8<XT>((uint32_t)src[0], (uint32_t)src[1]);
-    }
+    i32x4 xq[3];
+    xq[0] = xfrag(0);
+    xq[1] = xfrag(1);
     __builtin_amdgcn_sched_barrier(0);
-    constexpr int kEvery = MT / 4;  // a quarter of the next fragment after every kEvery th MFMA
-    qmm_static_for<4 * NG>([&](auto fc) {
-      constexpr int f = fc, j = f / NG, gi = f % NG;
-      constexpr bool kLastGroup = gi == NG - 1, kMore = f + 1 < 4 * NG;
-      constexpr int jn = kMore ? (f + 1) / NG : 0, gn = kMore ? (f + 1) % NG : 0;
-      i32x4 af_next = af;
-      qmm_static_for<MT>([&](auto mc) {
-        constexpr int mt = mc;
-        acc[gi][mt] = mfma16<XT>(af, xq[mt], acc[gi][mt]);
-        if constexpr (HASZP && kLastGroup) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[mt], xs[mt]);
-        if constexpr (kMore && mt % kEvery == 0) {
-          constexpr int q = mt / kEvery;  // element q of the fragment: bytes 2 (q & 1), 2 (q & 1) + 1 of dword q / 2
-          af_next[q] = (int)cvt_w2<XT>((uint32_t)wreg[(PH + (jn >> 1)) % H][gn][(jn & 1) * 2 + q / 2], qmm_const<(q & 1)>{});
+    constexpr int kEvery = MT / 4;  // a quarter of a fragment of the next j after every kEvery th MFMA
+    qmm_static_for<4 * MT>([&](auto ic) {
+      constexpr int idx = ic, j = idx / MT, mt = idx % MT, jn = j + 1;
+      if constexpr (idx + 2 < 4 * MT) xq[(idx + 2) % 3] = xfrag(idx + 2);
+      qmm_static_for<NG>([&](auto gc) {
+        constexpr int gi = gc, u = mt * NG + gi;
+        acc[gi][mt] = mfma16<XT>(af[j & 1][gi], xq[idx % 3], acc[gi][mt]);
+        if constexpr (HASZP && gi == NG - 1) xs[mt] = mfma16<XT>(ones_frag<XT>(), xq[idx % 3], xs[mt]);
+        if constexpr (u % kEvery == 0) {
+          // element q of fragment gn of the next j (of the next step's first j during the last one): bytes
+          // 2 (q & 1), 2 (q & 1) + 1 of dword q / 2 of its half's second or first 32 columns
+          constexpr int gn = (u / kEvery) / 4, q = (u / kEvery) % 4;
+          af[jn & 1][gn][q] = (int)cvt_w2<XT>((uint32_t)wreg[(PH + (jn >> 1)) % H][gn][(jn & 1) * 2 + q / 2], qmm_const<(q & 1)>{});
         }
-        if constexpr (kLastGroup && j + 1 < 4) xq[mt] = xfrag(j + 1, mt);
         __builtin_amdgcn_sched_barrier(0);
       });
-      if constexpr (kLastGroup && (j & 1)) {
+      // the half whose last fragments have just been converted (columns 0 .. 63 during j = 0, 64 .. 127 during j = 2)
+      if constexpr (mt == MT - 1 && (j & 1) == 0) {
         request(2 * s + (j >> 1) + H, last, qmm_const<(PH + (j >> 1)) % H>{});
         __builtin_amdgcn_sched_barrier(0);
       }
-      af = af_next;
     });
   };
 
@@ -482,6 +487,7 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
       xs[mt] = f32x4{0, 0, 0, 0};
       qmm_static_for<NG>([&](auto gc) { acc[(int)gc][mt] = f32x4{0, 0, 0, 0}; });
     });
+    prime();
     // H steps visit the H phases of the weight ring (step s starts at half 2 s, slot 2 s % H): unrolled, so that
     // every register of the ring is named at compile time; the last S % H steps follow one by one
     const int S = cur.steps;
