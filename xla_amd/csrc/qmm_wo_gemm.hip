@@ -387,14 +387,17 @@ qmm_wo_gemm_kernel(WoGemmArgs a) {
   const uint8_t* wp;     // wave-uniform: the first half block of the item in the tile's first channel group
   uint32_t w_lane[NG];   // from there to this lane's 16 bytes of row set gi (less than 2^32: 270 channels of K columns)
   i32x4 wreg[H][NG];     // ring: half q of the item (block q / 2, columns 64 (q % 2) ..) lives in slot q % H
+  // (divisions by G without a divide: the channel is at most 271 past the first channel of the tile's first
+  // group, and for t < 272 and G <= 16, t / G == (t * ceil(65536 / G)) >> 16)
+  const uint32_t g_magic = (65536u + (uint32_t)G - 1u) / (uint32_t)G;
   auto set_weights = [&](const WoItem& w) __attribute__((always_inline)) {
-    const int p0 = w.n0 / G;
+    const int p0 = w.n0 / G, a0 = w.n0 - p0 * G;
     wp = a.w + ((size_t)p0 * n_blk + w.k_begin / 128) * blk_bytes;
     qmm_static_for<NG>([&](auto gc) {
       constexpr int gi = gc;
-      const int ch = min(w.n0 + (wave * NG + gi) * 16 + r, N - 1);
-      const int p = ch / G, row = ch - p * G;
-      w_lane[gi] = (uint32_t)(p - p0) * ((uint32_t)n_blk * (uint32_t)blk_bytes) + (uint32_t)((g * G + row) * 16);
+      const uint32_t t = (uint32_t)(a0 + min((wave * NG + gi) * 16 + r, N - 1 - w.n0));
+      const uint32_t pd = (t * g_magic) >> 16, row = t - pd * (uint32_t)G;
+      w_lane[gi] = pd * ((uint32_t)n_blk * (uint32_t)blk_bytes) + ((uint32_t)(g * G) + row) * 16u;
     });
   };
   // half q of the item into its slot (a half past the end is the last one again: never used, and no branch
