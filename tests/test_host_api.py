@@ -340,7 +340,8 @@ def test_product_does_not_import_the_oracle():
 
 
 def test_fuse_quantized_linears_cpu():
-  # N-concatenated layers give exactly the outputs of the separate layers (CPU operator path)
+  # N-concatenated layers give the outputs of the separate layers (CPU operator path; to the last bits only: the
+  # host's matrix multiply may block a 48-column product differently from a 24-column one)
   import xla_amd.experimental.custom_kernel  # noqa: F401
   from xla_amd.quantization import quantize_linear, fuse_quantized_linears
   torch.manual_seed(3)
@@ -350,7 +351,7 @@ def test_fuse_quantized_linears_cpu():
     fused = fuse_quantized_linears(lins)
     outs = fused(x).split([l.output_dim for l in lins], dim=-1)
     for l, o in zip(lins, outs):
-      assert torch.equal(l(x), o), kwargs
+      torch.testing.assert_close(l(x), o, rtol=1e-5, atol=1e-6, msg=str(kwargs))
 
 
 def test_no_kernel_of_the_built_library_spills_registers():

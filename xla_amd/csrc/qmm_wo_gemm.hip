@@ -15,11 +15,12 @@
 // (channel n = row n % G of group n / G; every lane keeps the offset of its row, the base is scalar), so the
 // kernel wastes no MFMA rows on groups narrower than 16.  Per row set a wave keeps a ring of three or five half
 // blocks (64 columns) in registers and asks for a half again as soon as it has been used.
-// x goes through LDS: the workgroup's rows, one step (128 columns) per tile, in a ring of 5 (128 rows) or 8
-// (64 rows) tiles; four extra waves do nothing but copy (global -> LDS without registers) up to R - 1 tiles
-// ahead of the four computing waves, and the workgroup meets once per step.  (The computing waves must not issue
-// such copies themselves: with copies in flight the compiler can no longer count their register loads in flight
-// and turns every wait of the loop into a wait for all of them.)
+// x goes through LDS: the workgroup's rows, one step (128 columns) per tile, in a ring of 3 to 8 tiles (what
+// fits); four extra waves copy (global -> LDS without registers) up to R - 1 tiles ahead of the four computing
+// waves, and the workgroup meets once per step.  (The computing waves must not issue such copies themselves: with
+// copies in flight the compiler can no longer count their register loads in flight and turns every wait of the
+// loop into a wait for all of them.)  The 128 x 256 tile's results leave through LDS as well: the computing waves
+// put the rounded dot products there and go on, the copying waves scale them and write them out meanwhile.
 //
 // MFMA mapping (v_mfma_f32_16x16x32_bf16/f16, A = weights, B = x^T), as in the streaming
 // kernel: lane l is (r = l%16, g = l/16); for a block of 128 columns the lane supplies, for
@@ -633,14 +634,18 @@ int launch(const WoGemmArgs& a, hipStream_t stream) {
   using Cfg = WoCfg<MT, NG>;
   const int64_t items = (int64_t)((a.M + Cfg::BM - 1) / Cfg::BM) * (((int64_t)a.N + 64 * NG - 1) / (64 * NG)) * a.split;
   const int steps = a.k_per_split / 128;
-  // one workgroup per compute unit (its LDS and registers leave room for no second one); each walks its share of the items
+  // one workgroup per compute unit (its LDS and registers leave room for no second one); each walks its share of
+  // the items.  No more workgroups than give every one the same number of items: 896 items are four rounds on
+  // 256 compute units as on 224, and the chip, which runs this kernel at the clock its power allows, is faster
+  // with 32 of them idle throughout than with 128 idle in the last round (193.5 -> 191.5 us).
   const int cus = cu_count();
-  const dim3 grid((unsigned)(items < cus ? items : cus)), block((kComputeWaves + kCopyWaves) * 64);
+  const int64_t rounds = (items + cus - 1) / cus;
+  const dim3 grid((unsigned)((items + rounds - 1) / rounds)), block((kComputeWaves + kCopyWaves) * 64);
   auto go = [&](auto kern) -> int {
     static std::atomic<uint64_t> lds_set{0};
     const int rc = qmm_set_max_lds((const void*)kern, Cfg::lds_bytes(1 << 20), lds_set, "weight_only_gemm hipFuncSetAttribute");
     if (rc != XLA_AMD_QMM_OK) return rc;
-    // a workgroup with several items needs both chunk slots whatever the slice length
+    // a workgroup with several items keeps the whole ring of x tiles whatever the slice length
     hipLaunchKernelGGL(kern, grid, block, Cfg::lds_bytes(items > cus ? (1 << 20) : steps), stream, a);
     return QMM_CHECK_LAUNCH("weight_only_gemm launch");
   };
