@@ -760,9 +760,12 @@ size_t slice_workspace_floats(int slices, int64_t M, int64_t N, bool blockwise) 
   return blockwise ? 2 * mn : mn + (size_t)slices * (size_t)M;  // blockwise: room for the zero-point sums
 }
 
-// Tile and K split by shape.  Row tiles of 64 / 128 rows; 256 channels per workgroup
-// (128 when that is what fills the chip); K split over workgroups until about one workgroup
-// per compute unit is reached, in slices of at least 512 columns.
+// Tile and K split by shape.  Row tiles of 64 / 128 rows; 256 channels per workgroup, or 128 when the wide tiles
+// leave a quarter of the chip idle and the narrow ones still fit one round of workgroups (three row tiles against
+// 14336 channels: 168 wide tiles in one round take 48 us, 336 narrow ones in two rounds 59); K split over
+// workgroups while the items still fit one round (a part-full second round costs a whole one, and the second
+// kernel's partial sums grow with the split: 128 rows against 14336 x 4096 took 36 us in three slices, 336 items,
+// and take 28 in two), in slices of at least 512 columns.
 // (with a zero point the 128-row tile keeps 128 channels per workgroup: the row sums of x take
 // the registers that the wider tile would need)
 Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
@@ -771,11 +774,12 @@ Plan make_plan(int64_t M, int64_t N, int64_t K, bool has_zp) {
   const int64_t bm = 16 * p.mt;
   const int64_t tiles_m = (M + bm - 1) / bm;
   const int64_t groups = (N + 15) / 16;  // MFMA row sets of 16 channels: a column tile is 4 * ng of them
+  const int64_t wide = tiles_m * ((groups + 15) / 16), narrow = tiles_m * ((groups + 7) / 8);
   p.ng = 4;
-  if ((tiles_m * ((groups + 15) / 16) < 192 && N > 128) || (has_zp && p.mt == 8)) p.ng = 2;
-  const int64_t tiles = tiles_m * ((groups + 4 * p.ng - 1) / (4 * p.ng));
+  if ((wide < 192 && narrow <= 256 && N > 128) || (has_zp && p.mt == 8)) p.ng = 2;
+  const int64_t tiles = p.ng == 2 ? narrow : wide;
   int64_t split = 1;
-  if (tiles < 192) split = (256 + tiles - 1) / tiles;
+  if (tiles <= 128) split = 256 / tiles;
   const int64_t blocks = K / 128;
   int64_t per = (blocks + split - 1) / split;
   if (per < 4) per = blocks < 4 ? blocks : 4;
