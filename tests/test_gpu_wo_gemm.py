@@ -110,7 +110,12 @@ def test_blockwise_and_int4_gemm(ops, xdt):
   # several chunks, more tiles than compute units
   for (m, n, k, c, bits, asym) in [(65, 128, 256, 128, 8, False), (100, 200, 1024, 128, 4, True), (128, 4096, 4096, 128, 4, True),
                                    (130, 60, 1536, 512, 8, True), (300, 1000, 2048, 256, 4, False), (65, 4, 128, 128, 4, True),
-                                   (70, 132, 2560, 640, 8, False), (513, 8192, 1024, 128, 4, True)]:
+                                   (70, 132, 2560, 640, 8, False), (513, 8192, 1024, 128, 4, True),
+                                   # blocks of 128 columns (the kernel that rounds a block during the next one's MFMAs):
+                                   # 5 and 11 steps (an odd count, a last chunk of one and of three steps), int4 without
+                                   # and int8 with a zero point (the latter keeps the other kernel), several items
+                                   (90, 264, 640, 128, 4, False), (200, 136, 1408, 128, 8, False), (80, 128, 384, 128, 8, True),
+                                   (700, 5000, 1152, 128, 4, True)]:
     x, w, s, z, _ = cases.blockwise(m, n, k, c, bits, xdt, symmetric=not asym, seed=m + n)
     exp = oracle.quantized_matmul(x, w, s, z if asym else None, block_size=c, int4_weight=bits == 4)
     before = ops.counters["wo_gemm"]

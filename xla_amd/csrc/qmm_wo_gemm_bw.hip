@@ -49,7 +49,11 @@ struct BwItem {
   int m0, n0, rows;
 };
 
-template <int XT, int BITS, bool HASZP>
+// BLK1: quantization blocks of 128 columns, one per step.  The block's rounding sequence (some 180 of the step's 250
+// vector instructions) then runs a step late, between the MFMAs of the next block, which accumulate into a second
+// set of registers: a wave issues in order, so the MFMAs of a step only overlap with vector instructions that sit
+// between them in the instruction stream.
+template <int XT, int BITS, bool HASZP, bool BLK1>
 __global__ void __launch_bounds__((kComputeWaves + kCopyWaves) * 64)
 qmm_wo_bw_gemm_kernel(WoBwArgs a) {
   constexpr bool NEEDXS = HASZP || BITS == 4;        // block sums of x: zero point, int4 affine map
@@ -230,11 +234,218 @@ qmm_wo_bw_gemm_kernel(WoBwArgs a) {
     }
   };
 
+  // ---- results: four consecutive channels of one row per lane ----
+  auto store_results = [&](const BwItem& done) __attribute__((always_inline)) {
+  constexpr float kFactor = BITS == 4 ? 16.0f : 1.0f;
+  qmm_static_for<MT>([&](auto mc) {
+    constexpr int mt = mc;
+    const int m = done.m0 + 16 * mt + r;
+    qmm_static_for<NG>([&](auto gc) {
+      constexpr int gi = gc;
+      const int n = done.n0 + (wave * NG + gi) * 16 + 4 * g;
+      if (m < M && n < N) {  // N % 4 == 0: the four channels exist and the address is 8-byte aligned
+        float o[4];
+        qmm_static_for<4>([&](auto vc) {
+          constexpr int v = vc;
+          float t = qmm_round_dt(kFactor * sacc[gi][mt][v], XT);
+          if constexpr (HASZP) t = qmm_round_dt(t - qmm_round_dt(zacc[gi][mt][v], XT), XT);
+          o[v] = t;
+        });
+        uint32_t lo, hi;
+        if constexpr (XT == XLA_AMD_DT_BF16) {
+          lo = qmm_f32x2_to_bf16x2(o[0], o[1]); hi = qmm_f32x2_to_bf16x2(o[2], o[3]);
+        } else {
+          lo = qmm_f32x2_to_f16x2(o[0], o[1]); hi = qmm_f32x2_to_f16x2(o[2], o[3]);
+        }
+        *(i32x2*)((uint16_t*)a.out + (size_t)m * N + n) = i32x2{(int)lo, (int)hi};
+      }
+    });
+  });
+  };
   int it = blockIdx.x;
   BwItem cur = item_of(it);
   set_weights(cur);
   load_next(0);
   int ring = 0;
+
+  // ---- one block per step: the block's sums in two sets of registers, used in turn ----
+  f32x4 acc2[2][NG][MT], xs2[2][MT];
+  i32x2 ent_s[2][NG], ent_z[2][NG];  // scales and zero points of this lane's channels for the block in set P
+  // The rounding sequence of the block in set Q for the results (gi, v, mt) and (gi, v, mt + 1), in kPhases parts
+  // (one after each of kPhases consecutive MFMAs): the dot products rounded and packed; unpacked and added to the
+  // scaled sums; the zero-point sums.
+  float xs_r[MT];
+  uint32_t packed = 0;  // the pair's rounded dot products between the first and the second part
+  constexpr int kPairs = NG * 4 * (MT / 2);                 // pairs of results per block and lane
+  constexpr int kSlots = 4 * (NG * MT + (NEEDXS ? MT : 0));  // MFMAs per step
+  constexpr int kPhases = kSlots / kPairs;                  // MFMAs per pair
+  static_assert(MT % 2 == 0 && kSlots % kPairs == 0 && (kPhases == 2 || kPhases == 3), "the pairs spread evenly over the step's MFMAs");
+  auto block_pair = [&](auto qc, auto prc, auto phc) __attribute__((always_inline)) {
+    constexpr int Q = qc, pr = prc, ph = phc;  // pair (gi, v, mt): mt fastest
+    constexpr int gi = pr / (4 * (MT / 2)), v = (pr / (MT / 2)) % 4, mt = 2 * (pr % (MT / 2));
+    if constexpr (ph == 0) {
+      float d0 = acc2[Q][gi][mt][v], d1 = acc2[Q][gi][mt + 1][v];
+      if constexpr (BITS == 4) {  // (times 16, applied at the end)
+        d0 = fmaf(-1.5f, xs2[Q][mt][0], d0);
+        d1 = fmaf(-1.5f, xs2[Q][mt + 1][0], d1);
+      }
+      packed = XT == XLA_AMD_DT_BF16 ? qmm_f32x2_to_bf16x2(d0, d1) : qmm_f32x2_to_f16x2(d0, d1);
+    }
+    if constexpr (ph == 1) {
+      const uint32_t sw = (uint32_t)ent_s[Q][gi][v >> 1];
+      const float sc = qmm_from_raw((v & 1) ? (sw >> 16) : (sw & 0xffffu), XT);
+      const float p0 = qmm_from_raw(packed & 0xffffu, XT), p1 = qmm_from_raw(packed >> 16, XT);
+      sacc[gi][mt][v] = fmaf(sc, p0, sacc[gi][mt][v]);
+      sacc[gi][mt + 1][v] = fmaf(sc, p1, sacc[gi][mt + 1][v]);
+    }
+    if constexpr (HASZP && ph == kPhases - 1) {
+      const uint32_t zw = (uint32_t)ent_z[Q][gi][v >> 1];
+      const float zv = qmm_from_raw((v & 1) ? (zw >> 16) : (zw & 0xffffu), XT);
+      zacc[gi][mt][v] = fmaf(xs_r[mt], zv, zacc[gi][mt][v]);
+      zacc[gi][mt + 1][v] = fmaf(xs_r[mt + 1], zv, zacc[gi][mt + 1][v]);
+    }
+  };
+  auto block_sums_of_x = [&](auto qc) __attribute__((always_inline)) {
+    constexpr int Q = qc;
+    qmm_static_for<MT>([&](auto mc) { xs_r[(int)mc] = NEEDXS ? qmm_round_dt(xs2[Q][(int)mc][0], XT) : 0.f; });
+  };
+  // Constants of the int4 expansion and the fragment of ones kept in registers the compiler cannot see through: it
+  // would otherwise build the ones again for every j (two moves per MFMA against them), and with both constants of
+  // (x & mask) | one as literals it cannot use the single instruction for it.
+  i32x4 ones = ones_frag<XT>();
+  uint32_t k_one = XT == XLA_AMD_DT_BF16 ? 0x3F803F80u : 0x3C003C00u;
+  uint32_t k_mask = XT == XLA_AMD_DT_BF16 ? 0x00780078u : 0x03C003C0u;
+  asm volatile("" : "+v"(ones), "+v"(k_one), "+s"(k_mask));
+  // element q (two columns) of the fragment (j, gi) of the step's weights
+  auto frag_q = [&](auto jc, auto gic, auto qc) __attribute__((always_inline)) {
+    constexpr int j = jc, gi = gic, q = qc;
+    if constexpr (BITS == 8) {
+      return (int)cvt_w2<XT>((uint32_t)wcur[gi][j >> 1][(j & 1) * 2 + q / 2], qmm_const<(q & 1)>{});
+    } else {
+      const uint32_t d = (uint32_t)wcur[gi][0][j];
+      constexpr int sh = XT == XLA_AMD_DT_BF16 ? 4 * q - 3 : 4 * q - 6;  // right shift (negative: left)
+      const uint32_t t = sh < 0 ? d << (sh < 0 ? -sh : 0) : d >> (sh < 0 ? 0 : sh);
+      return (int)((t & k_mask) | k_one);
+    }
+  };
+  // One step = one block into set P, out of LDS tile `tile`, with the rounding sequence of the block in set 1 - P
+  // and the conversions of the step's own weights spread over its MFMAs.
+  auto step_blk1 = [&](int tile, auto pc) __attribute__((always_inline)) {
+    constexpr int P = pc, Q = 1 - P;
+    const char* xbase = xsm + tile * X_TILE;
+    qmm_static_for<NG>([&](auto gc) {
+      constexpr int gi = gc;
+      const char* ent = smem + tile * kEntryBytes + ((wave * NG + gi) * 16 + 4 * g) * 2;
+      ent_s[P][gi] = *(const i32x2*)ent;
+      if constexpr (HASZP) ent_z[P][gi] = *(const i32x2*)(ent + kSclTensor);
+      else ent_z[P][gi] = i32x2{0, 0};
+    });
+    i32x4 xq[MT];
+    qmm_static_for<MT>([&](auto mc) {
+      constexpr int mt = mc;
+      xq[mt] = *(const i32x4*)(xbase + (16 * mt + r) * 256 + (((4 * g + 0) ^ r) * 16));
+    });
+    i32x4 af, af_next;
+    qmm_static_for<4>([&](auto qc) { af[(int)qc] = frag_q(qmm_const<0>{}, qmm_const<0>{}, qc); });
+    af_next = af;
+    block_sums_of_x(qmm_const<Q>{});
+    __builtin_amdgcn_sched_barrier(0);
+    // after MFMA `slot` of the step: its share of the other block's rounding sequence
+    auto after = [&](auto slotc) __attribute__((always_inline)) {
+      constexpr int slot = slotc;
+      block_pair(qmm_const<Q>{}, qmm_const<slot / kPhases>{}, qmm_const<slot % kPhases>{});
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    constexpr int kPerJ = kSlots / 4;
+    static_assert(MT == 4, "a fragment has four elements: one is converted after each of the MT MFMAs of a fragment");
+    qmm_static_for<4>([&](auto jc) {
+      constexpr int j = jc;
+      qmm_static_for<NG>([&](auto gc) {
+        constexpr int gi = gc;
+        // the next fragment in the order (j, 0), (j, 1), .., (j + 1, 0): converted during this one's MFMAs, the first
+        // of the next j during the MFMAs against the ones (or, without them, during the last fragment of this j)
+        constexpr bool kConvHere = gi + 1 < NG || (!NEEDXS && j + 1 < 4);
+        constexpr int jn = gi + 1 < NG ? j : j + 1, gn = gi + 1 < NG ? gi + 1 : 0;
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          if constexpr (j == 0) acc2[P][gi][mt] = mfma16<XT>(af, xq[mt], f32x4{0, 0, 0, 0});
+          else acc2[P][gi][mt] = mfma16<XT>(af, xq[mt], acc2[P][gi][mt]);
+          if constexpr (kConvHere) af_next[mt] = frag_q(qmm_const<jn>{}, qmm_const<gn>{}, mc);
+          if constexpr (!NEEDXS && gi == NG - 1 && j + 1 < 4)
+            xq[mt] = *(const i32x4*)(xbase + (16 * mt + r) * 256 + (((4 * g + j + 1) ^ r) * 16));
+          after(qmm_const<j * kPerJ + gi * MT + mt>{});
+        });
+        if constexpr (kConvHere) af = af_next;
+      });
+      if constexpr (NEEDXS) {
+        qmm_static_for<MT>([&](auto mc) {
+          constexpr int mt = mc;
+          if constexpr (j == 0) xs2[P][mt] = mfma16<XT>(ones, xq[mt], f32x4{0, 0, 0, 0});
+          else xs2[P][mt] = mfma16<XT>(ones, xq[mt], xs2[P][mt]);
+          if constexpr (j + 1 < 4) {
+            af_next[mt] = frag_q(qmm_const<j + 1>{}, qmm_const<0>{}, mc);
+            xq[mt] = *(const i32x4*)(xbase + (16 * mt + r) * 256 + (((4 * g + j + 1) ^ r) * 16));
+          }
+          after(qmm_const<j * kPerJ + NG * MT + mt>{});
+        });
+        if constexpr (j + 1 < 4) af = af_next;
+      }
+    });
+  };
+  if constexpr (BLK1) {
+    for (;;) {
+      qmm_static_for<MT>([&](auto mc) {
+        constexpr int mt = mc;
+        xs2[1][mt] = f32x4{0, 0, 0, 0};
+        qmm_static_for<NG>([&](auto gc) {
+          sacc[(int)gc][mt] = f32x4{0, 0, 0, 0};
+          zacc[(int)gc][mt] = f32x4{0, 0, 0, 0};
+          acc2[1][(int)gc][mt] = f32x4{0, 0, 0, 0};
+        });
+      });
+      // (the first step's rounding sequence runs over zeros: a scale of 0 and sums of 0 add nothing)
+      qmm_static_for<NG>([&](auto gc) { ent_s[1][(int)gc] = i32x2{0, 0}; ent_z[1][(int)gc] = i32x2{0, 0}; });
+      int s = 0;
+      for (int c = 0; c < n_chunks; ++c, ++ring) {
+        qmm_bare_barrier();  // chunk `ring` is there (the copying waves waited for it)
+        const int tile0 = (ring & 1) * CS - c * CS;
+        const int s_end = min(steps, (c + 1) * CS);
+        static_assert(CS % 2 == 0, "a chunk begins with set 0");
+        qmm_static_for<CS>([&](auto kc) {
+          if (s < s_end) {
+            qmm_static_for<NG>([&](auto gc) {
+              qmm_static_for<WL>([&](auto hc) { wcur[(int)gc][(int)hc] = wnext[(int)gc][(int)hc]; });
+            });
+            if (s + 1 < steps) load_next(s + 1);
+            step_blk1(tile0 + s, qmm_const<(int)kc % 2>{});
+            ++s;
+          }
+        });
+      }
+      const BwItem done = cur;
+      const int it_next = it + (int)gridDim.x;
+      const bool more = it_next < n_items;
+      if (more) {
+        it = it_next;
+        cur = item_of(it);
+        set_weights(cur);
+        load_next(0);
+      }
+      // the last block's rounding sequence: it is in set 1 after an even number of steps, else in set 0
+      auto last_block = [&](auto qc) __attribute__((always_inline)) {
+        block_sums_of_x(qc);
+        qmm_static_for<kPairs>([&](auto prc) {
+          qmm_static_for<kPhases>([&](auto phc) { block_pair(qc, prc, phc); });
+        });
+      };
+      if (steps & 1) last_block(qmm_const<0>{});
+      else last_block(qmm_const<1>{});
+      store_results(done);
+      if (!more) break;
+    }
+    return;
+  }
+
   for (;;) {
     qmm_static_for<MT>([&](auto mc) {
       constexpr int mt = mc;
@@ -271,32 +482,7 @@ qmm_wo_bw_gemm_kernel(WoBwArgs a) {
       load_next(0);
     }
 
-    // ---- results: four consecutive channels of one row per lane ----
-    constexpr float kFactor = BITS == 4 ? 16.0f : 1.0f;
-    qmm_static_for<MT>([&](auto mc) {
-      constexpr int mt = mc;
-      const int m = done.m0 + 16 * mt + r;
-      qmm_static_for<NG>([&](auto gc) {
-        constexpr int gi = gc;
-        const int n = done.n0 + (wave * NG + gi) * 16 + 4 * g;
-        if (m < M && n < N) {  // N % 4 == 0: the four channels exist and the address is 8-byte aligned
-          float o[4];
-          qmm_static_for<4>([&](auto vc) {
-            constexpr int v = vc;
-            float t = qmm_round_dt(kFactor * sacc[gi][mt][v], XT);
-            if constexpr (HASZP) t = qmm_round_dt(t - qmm_round_dt(zacc[gi][mt][v], XT), XT);
-            o[v] = t;
-          });
-          uint32_t lo, hi;
-          if constexpr (XT == XLA_AMD_DT_BF16) {
-            lo = qmm_f32x2_to_bf16x2(o[0], o[1]); hi = qmm_f32x2_to_bf16x2(o[2], o[3]);
-          } else {
-            lo = qmm_f32x2_to_f16x2(o[0], o[1]); hi = qmm_f32x2_to_f16x2(o[2], o[3]);
-          }
-          *(i32x2*)((uint16_t*)a.out + (size_t)m * N + n) = i32x2{(int)lo, (int)hi};
-        }
-      });
-    });
+    store_results(done);
     if (!more) break;
   }
 }
@@ -326,7 +512,13 @@ int launch(const WoBwArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL(kern, grid, block, kLdsBytes, stream, a);
     return QMM_CHECK_LAUNCH("weight_only_gemm (blockwise) launch");
   };
-  return a.zp ? go(qmm_wo_bw_gemm_kernel<XT, BITS, true>) : go(qmm_wo_bw_gemm_kernel<XT, BITS, false>);
+  // blocks of 128 columns: the kernel with two sets of block sums (int8 weights with a zero point keep the other
+  // one: their two 16-byte weight loads per row set leave no registers for the second set)
+  if (a.C == 128) {
+    if (!a.zp) return go(qmm_wo_bw_gemm_kernel<XT, BITS, false, true>);
+    if constexpr (BITS == 4) return go(qmm_wo_bw_gemm_kernel<XT, BITS, true, true>);
+  }
+  return a.zp ? go(qmm_wo_bw_gemm_kernel<XT, BITS, true, false>) : go(qmm_wo_bw_gemm_kernel<XT, BITS, false, false>);
 }
 
 }  // namespace
