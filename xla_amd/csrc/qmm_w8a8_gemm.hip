@@ -187,44 +187,64 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
 
   const int lrow = lane & 31, lchunk = lane >> 5;
-  // One K step out of LDS: 4 sub-steps of 32 bytes.  The operand fragments of
-  // sub-step ks+1 are read while the MFMAs of sub-step ks run (two register
-  // sets), so the matrix pipe does not wait for LDS latency between sub-steps.
-  auto compute = [&](int stage, auto&& after_first_reads) __attribute__((always_inline)) {
+  // Copy `piece` (a 1 KB slice of this wave: A slices first) of a whole step into `stage`.
+  auto copy_piece = [&](int stage, int k0, auto pc) __attribute__((always_inline)) {
+    constexpr int p = pc;
+    if constexpr (p < A_CH)
+      __builtin_amdgcn_global_load_lds((const void*)(ga[p] + k0), (lds_ptr_t)(sA + stage * BM * kBK + wave * 1024 + p * (T * 16)), 16, 0, 0);
+    else
+      __builtin_amdgcn_global_load_lds((const void*)(gb[p - A_CH] + k0), (lds_ptr_t)(sB + stage * BN * kBK + wave * 1024 + (p - A_CH) * (T * 16)), 16, 0, 0);
+  };
+  // One K step out of LDS: 4 sub-steps of 32 bytes.  The operand fragments of sub-step ks+1 are read while the
+  // MFMAs of sub-step ks run (two register sets), one read after each MFMA, and the copies of the step NS - 1
+  // ahead are issued the same way, one after each of the step's first MFMAs.  A wave issues in order: issued as
+  // a run (6 reads before a sub-step's MFMAs, 8 copies with their addresses at the start of the step) they keep
+  // the wave from issuing MFMAs for that long, and the two waves of a SIMD, which leave the step's barrier
+  // together, do it at the same moment.
+  // COPY: 0 = no copies, 1 = a whole step (spread), 2 = the last, partial step (as a run: its chunks past K are
+  // zero-filled under per-lane conditions).
+  auto compute = [&](int stage, int COPY, int cstage, int ck0) __attribute__((always_inline)) {
     const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
     const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
     i32x4 af[2][MI], bf[2][NI];
-    auto read_frags = [&](auto setc, auto ksc) __attribute__((always_inline)) {
-      constexpr int set = setc, ks = ksc;
+    auto read_frag = [&](auto setc, auto ksc, auto nc) __attribute__((always_inline)) {  // fragment n: A tiles, then B tiles
+      constexpr int set = setc, ks = ksc, n = nc;
       const int c = 2 * ks + lchunk;
-      qmm_static_for<MI>([&](auto ic) {
-        constexpr int i = ic;
-        const int row = i * 32 + lrow;
-        af[set][i] = *(const i32x4*)(a_base + row * kBK + swz(wm * TM + row, c) * 16);
-      });
-      qmm_static_for<NI>([&](auto jc) {
-        constexpr int j = jc;
-        const int row = j * 32 + lrow;
-        bf[set][j] = *(const i32x4*)(b_base + row * kBK + swz(wn * TN + row, c) * 16);
-      });
+      if constexpr (n < MI) {
+        const int row = n * 32 + lrow;
+        af[set][n] = *(const i32x4*)(a_base + row * kBK + swz(wm * TM + row, c) * 16);
+      } else {
+        const int row = (n - MI) * 32 + lrow;
+        bf[set][n - MI] = *(const i32x4*)(b_base + row * kBK + swz(wn * TN + row, c) * 16);
+      }
     };
-    read_frags(qmm_const<0>{}, qmm_const<0>{});
+    qmm_static_for<MI + NI>([&](auto nc) { read_frag(qmm_const<0>{}, qmm_const<0>{}, nc); });
     __builtin_amdgcn_sched_barrier(0);
-    after_first_reads();  // the next stage's copies are issued while those reads are in flight
+    if (COPY == 2) stage_load(cstage, ck0);
+    constexpr int kPerSub = MI * NI;
     qmm_static_for<kBK / 32>([&](auto ksc) {
       constexpr int ks = ksc, set = ks & 1;
-      if constexpr (ks + 1 < kBK / 32) read_frags(qmm_const<set ^ 1>{}, qmm_const<ks + 1>{});
-      // keep those reads ahead of this sub-step's MFMAs (the scheduler would
-      // otherwise sink each read next to its first use to save registers)
-      __builtin_amdgcn_sched_barrier(0);
+      constexpr bool kMore = ks + 1 < kBK / 32;
       qmm_static_for<MI>([&](auto ic) {
         constexpr int i = ic;
         qmm_static_for<NI>([&](auto jc) {
-          constexpr int j = jc;
+          constexpr int j = jc, n = i * NI + j, at = ks * kPerSub + n;
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+          if constexpr (kMore && n < MI + NI) read_frag(qmm_const<set ^ 1>{}, qmm_const<ks + 1>{}, qmm_const<n>{});
+          if constexpr (at < kStageOps) { if (COPY == 1) copy_piece(cstage, ck0, qmm_const<at>{}); }
+          __builtin_amdgcn_sched_barrier(0);
         });
       });
+      // (tiles with fewer MFMAs than fragments per sub-step: the rest of the reads)
+      if constexpr (kMore && kPerSub < MI + NI) {
+        qmm_static_for<MI + NI - kPerSub>([&](auto nc) { read_frag(qmm_const<set ^ 1>{}, qmm_const<ks + 1>{}, qmm_const<kPerSub + (int)nc>{}); });
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
+    if constexpr ((kBK / 32) * kPerSub < kStageOps) {
+      if (COPY == 1)
+        qmm_static_for<kStageOps - (kBK / 32) * kPerSub>([&](auto pc) { copy_piece(cstage, ck0, qmm_const<(kBK / 32) * kPerSub + (int)pc>{}); });
+    }
   };
 
   // Steps 0 .. NS-2 are copied ahead; step kt then computes stage kt % NS while the
@@ -245,10 +265,10 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   int cur = 0, nxt = NS - 1;
   for (int kt = 0; kt < kiters; ++kt) {
     stage_sync(kt + NS - 2 < ksteps - 1);
-    if (KG == 1 || kt < ksteps)
-      compute(cur, [&]() __attribute__((always_inline)) {
-        if (kt + NS - 1 < ksteps) stage_load(nxt, step_k0(kt + NS - 1));
-      });
+    if (KG == 1 || kt < ksteps) {
+      const int ck0 = step_k0(kt + NS - 1);
+      compute(cur, kt + NS - 1 >= ksteps ? 0 : ck0 + kBK <= K ? 1 : 2, nxt, ck0);
+    }
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
   }
