@@ -203,6 +203,11 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
   // together, do it at the same moment.
   // COPY: 0 = no copies, 1 = a whole step (spread), 2 = the last, partial step (as a run: its chunks past K are
   // zero-filled under per-lane conditions).
+  // Tiles with few MFMAs per step are bound by the latency of their copies and keep the runs (compute_runs below:
+  // the copies go out at once, as early as possible; 32 x 32 tiles at M = 32 against 4096 x 14336 take 15.2 us so
+  // and 16.6 - 18.7 us with any part of this order).
+  constexpr int kPerSub = MI * NI;
+  constexpr bool kSpread = kStageOps <= 2 * kPerSub;
   auto compute = [&](int stage, int COPY, int cstage, int ck0) __attribute__((always_inline)) {
     const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
     const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
@@ -221,7 +226,6 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
     qmm_static_for<MI + NI>([&](auto nc) { read_frag(qmm_const<0>{}, qmm_const<0>{}, nc); });
     __builtin_amdgcn_sched_barrier(0);
     if (COPY == 2) stage_load(cstage, ck0);
-    constexpr int kPerSub = MI * NI;
     qmm_static_for<kBK / 32>([&](auto ksc) {
       constexpr int ks = ksc, set = ks & 1;
       constexpr bool kMore = ks + 1 < kBK / 32;
@@ -241,10 +245,43 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
       }
     });
-    if constexpr ((kBK / 32) * kPerSub < kStageOps) {
-      if (COPY == 1)
-        qmm_static_for<kStageOps - (kBK / 32) * kPerSub>([&](auto pc) { copy_piece(cstage, ck0, qmm_const<(kBK / 32) * kPerSub + (int)pc>{}); });
-    }
+  };
+
+  auto compute_runs = [&](int stage, auto&& after_first_reads) __attribute__((always_inline)) {
+    const char* a_base = sA + stage * BM * kBK + (wm * TM) * kBK;
+    const char* b_base = sB + stage * BN * kBK + (wn * TN) * kBK;
+    i32x4 af[2][MI], bf[2][NI];
+    auto read_frags = [&](auto setc, auto ksc) __attribute__((always_inline)) {
+      constexpr int set = setc, ks = ksc;
+      const int c = 2 * ks + lchunk;
+      qmm_static_for<MI>([&](auto ic) {
+        constexpr int i = ic;
+        const int row = i * 32 + lrow;
+        af[set][i] = *(const i32x4*)(a_base + row * kBK + swz(wm * TM + row, c) * 16);
+      });
+      qmm_static_for<NI>([&](auto jc) {
+        constexpr int j = jc;
+        const int row = j * 32 + lrow;
+        bf[set][j] = *(const i32x4*)(b_base + row * kBK + swz(wn * TN + row, c) * 16);
+      });
+    };
+    read_frags(qmm_const<0>{}, qmm_const<0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    after_first_reads();  // the next stage's copies are issued while those reads are in flight
+    qmm_static_for<kBK / 32>([&](auto ksc) {
+      constexpr int ks = ksc, set = ks & 1;
+      if constexpr (ks + 1 < kBK / 32) read_frags(qmm_const<set ^ 1>{}, qmm_const<ks + 1>{});
+      // keep those reads ahead of this sub-step's MFMAs (the scheduler would
+      // otherwise sink each read next to its first use to save registers)
+      __builtin_amdgcn_sched_barrier(0);
+      qmm_static_for<MI>([&](auto ic) {
+        constexpr int i = ic;
+        qmm_static_for<NI>([&](auto jc) {
+          constexpr int j = jc;
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+        });
+      });
+    });
   };
 
   // Steps 0 .. NS-2 are copied ahead; step kt then computes stage kt % NS while the
@@ -267,7 +304,13 @@ qmm_w8a8_gemm_kernel(GemmArgs g) {
     stage_sync(kt + NS - 2 < ksteps - 1);
     if (KG == 1 || kt < ksteps) {
       const int ck0 = step_k0(kt + NS - 1);
-      compute(cur, kt + NS - 1 >= ksteps ? 0 : ck0 + kBK <= K ? 1 : 2, nxt, ck0);
+      if constexpr (kSpread) {
+        compute(cur, kt + NS - 1 >= ksteps ? 0 : ck0 + kBK <= K ? 1 : 2, nxt, ck0);
+      } else {
+        compute_runs(cur, [&]() __attribute__((always_inline)) {
+          if (kt + NS - 1 < ksteps) stage_load(nxt, ck0);
+        });
+      }
     }
     cur = cur + 1 == NS ? 0 : cur + 1;
     nxt = nxt + 1 == NS ? 0 : nxt + 1;
